@@ -1,0 +1,101 @@
+"""The step function and what it stands on: model, weights, cache, step arena.
+
+``ModelRunner.forward_step(rows)`` is the one way tokens become logits: generation
+(LLMEngine.step), trace replay and the benchmarks all call it.  It runs only the
+tokens it is given, as one flattened batch, against the cache earlier steps left,
+and returns 32-bit logits at the wanted places in the caller's order.  (The
+reference's counterpart is LLMEngine._prepare + LlamaModel.forward,
+inference_engine/engine.py:133-201, which returns logits for the last token of
+finished prompts only.)
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache import CacheManager, CacheStorage, GroupSpec
+from ..config.registry import architecture_of, load_model_config
+from ..models.decoder import Decoder
+from ..weights import load_weights
+from .batch import StepArena, StepRow, build_step
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def parse_dtype(d) -> torch.dtype:
+    if d not in _DTYPES:
+        raise ValueError(f"dtype {d!r}: choose bfloat16 or float32")
+    return _DTYPES[d]
+
+
+class ModelRunner:
+    def __init__(self, model, *, dtype=torch.bfloat16, device="cuda", backend=None, page_size: int = 16,
+                 num_pages: int | None = None, memory_fraction: float = 0.85, reserve_bytes: int = 768 * 2**20,
+                 max_step_tokens: int = 2048, max_rows: int = 256, max_model_len: int | None = None,
+                 num_state_slots: int | None = None, weights=None):
+        """``model``: a folder with config.json and safetensors, or a ModelConfig together
+        with ``weights`` (name -> tensor).  ``backend``: the kernels; by default the HIP
+        library, which must load (there is no other product path)."""
+        self.dtype = parse_dtype(dtype)
+        self.device = torch.device(device)
+        if isinstance(model, str):
+            self.model_cfg, arch = load_model_config(model)
+            source = model
+        else:
+            self.model_cfg, arch = model, architecture_of(model)
+            if weights is None:
+                raise ValueError("a configuration needs weights (name -> tensor) beside it")
+            source = weights
+        self.model = Decoder(arch.build(self.model_cfg))
+        if backend is None:
+            from ..kernels.hip_backend import HipBackend
+            backend = HipBackend(self.dtype, self.device)
+        self.ops = backend
+        self.model.use_backend(backend)
+        self.load_report = load_weights(self.model, source, self.device, self.dtype)
+        self.model.prepare(self.device, self.dtype)
+
+        spec = self.model.spec
+        limit = spec.max_position or (1 << 30)
+        self.max_model_len = min(max_model_len or limit, limit)
+        self.page_size = page_size
+        self.max_blocks = -(-self.max_model_len // page_size)
+        elem = 2 if self.dtype == torch.bfloat16 else 4
+        per_page = self.model.bytes_per_page(page_size, elem)
+        n_groups = len(per_page)
+        if num_pages is None:
+            if self.device.type != "cuda":
+                raise ValueError("num_pages must be given off the GPU")
+            torch.cuda.empty_cache()
+            free, _ = torch.cuda.mem_get_info(self.device)
+            budget = int((free - reserve_bytes) * memory_fraction)
+            num_pages = max(2, budget // max(1, sum(per_page))) if n_groups else 2
+        self.num_pages = int(num_pages)
+        self.num_state_slots = int(num_state_slots or max_rows + 1)
+        self.cache = CacheManager(page_size, [GroupSpec(w, self.num_pages) for w in self.model.page_groups],
+                                  self.num_state_slots)
+        self.storage = CacheStorage(self.model, page_size, [self.num_pages] * n_groups, self.num_state_slots,
+                                    self.device, self.dtype)
+        self.model.attach_cache(self.storage)
+        self.arena = StepArena(max_step_tokens, max_rows, self.max_blocks, n_groups, self.device)
+        self.vocab_size = spec.vocab_size
+
+    # ------------------------------------------------------------------ steps
+    def build(self, rows: list[StepRow], **kw):
+        for r in rows:
+            if r.start + len(r.tokens) > self.max_model_len:
+                raise ValueError(f"a row reaches position {r.start + len(r.tokens)}, beyond max_model_len "
+                                 f"{self.max_model_len}")
+        return build_step(rows, self.arena, self.page_size, **kw)
+
+    @torch.inference_mode()
+    def forward_step(self, rows: list[StepRow]) -> torch.Tensor | None:
+        """Logits [sum of wants, vocab] float32, ordered by row then by ``want``.
+        Pages for the rows' tokens must have been reserved."""
+        step = self.build(rows)
+        return self.model.forward(step)
+
+    def after_step(self, rows: list[StepRow]) -> None:
+        """Tell the cache how far each row's request has come (windows release pages)."""
+        for r in rows:
+            self.cache.advance(r.cache, r.start + len(r.tokens))

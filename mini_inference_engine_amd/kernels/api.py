@@ -1,0 +1,55 @@
+"""The operations parts compute with.  The product has one implementation, the
+HIP library (hip_backend.HipBackend); tests hand a model another one to check
+the engine's host logic without a GPU.
+
+Conventions: T tokens of a step, flattened; activations in ``act_dtype``
+(bfloat16 or float32); the residual stream and logits in float32; int32 indices.
+Every op runs on the current stream and allocates its outputs with torch.
+"""
+from __future__ import annotations
+
+
+class KernelBackend:
+    name = "?"
+    act_dtype = None
+
+    def embedding(self, ids, table):
+        """stream[t, :] = float(table[ids[t], :]) -> [T, width] float32."""
+        raise NotImplementedError
+
+    def add_rmsnorm(self, x, residual, weight, eps, out_dtype=None, rows=None):
+        """If ``x`` is given: residual += float(x), in place.  y = residual *
+        rsqrt(mean(residual^2) + eps) * weight, all in float32, rounded once to
+        ``out_dtype`` (default act_dtype).  With ``rows`` only those rows are
+        computed, y is [len(rows), width] and residual is not modified."""
+        raise NotImplementedError
+
+    def linear(self, x, w, bias=None, out_dtype=None):
+        """y = x w^T (+ bias); w [out, in]; 32-bit accumulation."""
+        raise NotImplementedError
+
+    def linear_silu_mul(self, x, w_gate_up, intermediate):
+        """gu = x w^T with w [2 * intermediate, in]; returns silu(gu[:, :I]) * gu[:, I:]."""
+        raise NotImplementedError
+
+    def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
+                        k_cache, v_cache, slot_mapping):
+        """Rotate the first ``rotary_dim`` dims of every q and k head of
+        qkv [T, (Hq + 2 Hkv) D] in place (pairs j, j + rotary_dim / 2; angle tables
+        cos, sin [positions, rotary_dim / 2] float32), then write k and v of token t to
+        cache slot slot_mapping[t] of k_cache, v_cache [pages, Hkv, page, D].
+        rotary_dim 0: no rotation.  num_kv_heads 0 (k_cache None): q only, no write."""
+        raise NotImplementedError
+
+    def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
+                        window):
+        """For token t of row r at position p: softmax over keys max(0, p - window + 1)..p
+        of row r (read through group.block_tables[r]) of (q . k) * scale, times v.
+        q head i uses kv head i // (Hq / Hkv).  q is the first Hq * D columns of
+        qkv (row stride qkv.stride(0)).  Returns [T, Hq * D] in act_dtype."""
+        raise NotImplementedError
+
+    def sample(self, logits, temperatures, seeds, counters):
+        """Per row: argmax(logits) if temperature == 0, else argmax(logits / temperature + g)
+        with Gumbel noise g from (seed, counter, vocabulary index).  -> [R] int32."""
+        raise NotImplementedError

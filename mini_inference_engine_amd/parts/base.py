@@ -1,0 +1,223 @@
+"""Interfaces of the parts a decoder is put together from.
+
+A part owns its sizes and constants as constructor parameters, declares the
+checkpoint tensors it wants (``params``), says what cache it needs
+(``cache_requirement``, mixers only) and computes through a kernel backend
+(``self.ops``) that the model hands to every part.  No part knows which model
+it is in, which layer it is, or what the other layers are.
+
+Interfaces
+----------
+Norm.forward(x, residual, rows=None) -> y
+    ``residual`` is the fp32 stream [T, width]; ``x`` (or None) is the branch
+    output still to be added to it.  Adds in place, normalises, returns ``y`` in
+    the activation dtype.  With ``rows`` (int32 indices) only those rows are
+    produced and the stream is left untouched.
+PositionEncoding.encode_and_store(ops, qkv, step, layout, cache, slots)
+    Encodes q and k inside the fused projection output in place, as a function of
+    each token's absolute position only, and writes k, v to the cache.
+Mixer.forward(x, step, cache) -> y      [T, width] -> [T, width]
+    Must accept a portion that starts anywhere in a request and leave its cache
+    or state as if the request had been fed whole.
+FeedForward.forward(x, step) -> y       token-wise
+Block.forward(h, residual, step, cache) -> (h, residual)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Sequence
+
+
+@dataclass(frozen=True)
+class Source:
+    """One checkpoint tensor and where its rows go inside a (possibly fused) buffer."""
+    name: str
+    shape: tuple
+    row_offset: int = 0
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """A device buffer a part wants filled: one source, or several stacked on dim 0."""
+    attr: str
+    shape: tuple
+    sources: tuple
+    integer: bool = False   # integer tables are kept as int32
+
+    @staticmethod
+    def single(attr: str, name: str, shape: Sequence[int], integer: bool = False) -> "ParamSpec":
+        shape = tuple(int(s) for s in shape)
+        return ParamSpec(attr, shape, (Source(name, shape, 0),), integer)
+
+    @staticmethod
+    def stacked(attr: str, pieces: Sequence[tuple]) -> "ParamSpec":
+        """pieces: (name, shape) in row order; all share the trailing dims."""
+        sources, off = [], 0
+        tail = tuple(pieces[0][1][1:])
+        for name, shape in pieces:
+            shape = tuple(int(s) for s in shape)
+            if tuple(shape[1:]) != tail:
+                raise ValueError(f"cannot stack {name} {shape} on tail {tail}")
+            sources.append(Source(name, shape, off))
+            off += shape[0]
+        return ParamSpec(attr, (off,) + tail, tuple(sources))
+
+
+class Part:
+    """Base of all parts: parameter declaration, children, backend injection."""
+
+    ops: Any = None
+
+    def params(self) -> list[ParamSpec]:
+        return []
+
+    def children(self) -> list["Part"]:
+        return []
+
+    def walk(self):
+        yield self
+        for c in self.children():
+            yield from c.walk()
+
+    def bind(self, attr: str, tensor) -> None:
+        setattr(self, attr, tensor)
+
+    def prepare(self, device, dtype) -> None:
+        """Build derived device tables (none by default)."""
+
+    def use_backend(self, ops) -> None:
+        for p in self.walk():
+            p.ops = ops
+
+
+# ---------------------------------------------------------------- cache needs
+@dataclass(frozen=True)
+class PagedKV:
+    """Keys and values of every token in pages; ``window`` keys back at most, or all."""
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class FixedState:
+    """Per-request state of fixed size, indexed by the request's state slot.
+    ``dtype``: 'float32' or 'activation'."""
+    shape: tuple
+    dtype: str = "float32"
+
+
+@dataclass
+class CacheBinding:
+    """What a mixer call gets: the tensors of the cache entry it reads/writes."""
+    group: int | None = None          # page group id (PagedKV) or None
+    k: Any = None                     # [pages, kv_heads, page, head_dim]
+    v: Any = None
+    state: Any = None                 # [slots, *shape]
+    read_only: bool = False           # entry belongs to another layer call
+    page_size: int = 0
+
+
+class Norm(Part):
+    width: int
+
+    def forward(self, x, residual, rows=None):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    pass
+
+
+class Mixer(Part):
+    def cache_requirement(self):
+        return None
+
+    def forward(self, x, step, cache: CacheBinding):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, step):
+        raise NotImplementedError
+
+
+class Block(Part):
+    mixer: Mixer
+
+    def forward(self, h, residual, step, cache: CacheBinding):
+        raise NotImplementedError
+
+
+# ------------------------------------------------------------ part registries
+# Kind name -> class, so that a configuration can choose a part layer by layer
+# and a new kind can be added from outside the package.
+MIXERS: dict[str, type] = {}
+FEED_FORWARDS: dict[str, type] = {}
+NORMS: dict[str, type] = {}
+POSITION_ENCODINGS: dict[str, type] = {}
+BLOCKS: dict[str, type] = {}
+
+
+def _register(table: dict, kind: str):
+    def deco(cls):
+        table[kind] = cls
+        cls.kind = kind
+        return cls
+    return deco
+
+
+def register_mixer(kind: str):
+    return _register(MIXERS, kind)
+
+
+def register_feed_forward(kind: str):
+    return _register(FEED_FORWARDS, kind)
+
+
+def register_norm(kind: str):
+    return _register(NORMS, kind)
+
+
+def register_position_encoding(kind: str):
+    return _register(POSITION_ENCODINGS, kind)
+
+
+def register_block(kind: str):
+    return _register(BLOCKS, kind)
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    """One entry of the run order: which layer runs, and whose cache it uses.
+    ``cache_of`` names an earlier entry of the run order whose cache this call
+    reads instead of owning one."""
+    layer: int
+    cache_of: int | None = None
+
+
+@dataclass
+class DecoderSpec:
+    """A whole model as data: parts plus the order in which layers run."""
+    embedding: Part
+    layers: list
+    final_norm: Norm
+    head: Part
+    schedule: list = field(default_factory=list)
+    ignore_tensors: tuple = ()      # regular expressions of checkpoint names to skip
+    eos_token_id: int | None = None
+    max_position: int | None = None
+    vocab_size: int = 0
+
+    def __post_init__(self):
+        if not self.schedule:
+            self.schedule = [LayerCall(i) for i in range(len(self.layers))]
+        owners = set()
+        for e, call in enumerate(self.schedule):
+            if not 0 <= call.layer < len(self.layers):
+                raise ValueError(f"run order entry {e} names layer {call.layer}; there are {len(self.layers)}")
+            if call.cache_of is None:
+                owners.add(e)
+            elif call.cache_of not in owners or call.cache_of >= e:
+                raise ValueError(f"run order entry {e} reads the cache of entry {call.cache_of}, "
+                                 "which must be an earlier entry that owns one")

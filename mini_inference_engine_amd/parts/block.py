@@ -1,0 +1,28 @@
+"""Pre-norm block with the residual adds deferred into the norms.
+
+stream += pending; y = norm1(stream); a = mixer(y); stream += a; y = norm2(stream);
+pending' = feed_forward(y).  The block returns its feed-forward output still to
+be added: the next block's first norm (or the final norm) adds it
+(inference_engine/model.py:169-171,179,184).
+"""
+from __future__ import annotations
+
+from .base import Block, register_block
+
+
+@register_block("pre_norm")
+class PreNormBlock(Block):
+    def __init__(self, norm_mixer, mixer, norm_feed_forward, feed_forward):
+        self.norm_mixer = norm_mixer
+        self.mixer = mixer
+        self.norm_feed_forward = norm_feed_forward
+        self.feed_forward = feed_forward
+
+    def children(self):
+        return [self.norm_mixer, self.mixer, self.norm_feed_forward, self.feed_forward]
+
+    def forward(self, h, residual, step, cache):
+        y = self.norm_mixer.forward(h, residual)
+        a = self.mixer.forward(y, step, cache)
+        y = self.norm_feed_forward.forward(a, residual)
+        return self.feed_forward.forward(y, step), residual

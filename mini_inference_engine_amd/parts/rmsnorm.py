@@ -1,0 +1,25 @@
+"""RMSNorm with the residual add folded in.
+
+y = weight * x * rsqrt(mean(x^2) + eps), taken of the stream after the pending
+branch output has been added to it (inference_engine/kernels/rmsnorm.py:56-65;
+used at inference_engine/model.py:171,179,184).  The weight is a plain multiplier.
+The stream and every intermediate are 32-bit; y is rounded once.
+"""
+from __future__ import annotations
+
+from .base import Norm, ParamSpec, register_norm
+
+
+@register_norm("rmsnorm")
+class RMSNorm(Norm):
+    def __init__(self, width: int, eps: float, weight_name: str):
+        self.width = int(width)
+        self.eps = float(eps)
+        self.weight_name = weight_name
+        self.weight = None
+
+    def params(self):
+        return [ParamSpec.single("weight", self.weight_name, (self.width,))]
+
+    def forward(self, x, residual, rows=None, out_dtype=None):
+        return self.ops.add_rmsnorm(x, residual, self.weight, self.eps, out_dtype=out_dtype, rows=rows)

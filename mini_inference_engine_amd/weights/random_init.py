@@ -1,0 +1,45 @@
+"""Random weights: a model folder (config.json, model.safetensors) from a
+configuration and a seed.  The reference has no such mode; the folder goes
+through the same loader a real checkpoint does.
+
+Matrices and embeddings are N(0, std), vectors (norm weights) 1 + N(0, std),
+drawn in float32 from one seeded CPU generator in the order the parts declare
+their tensors, then stored in the asked dtype.
+"""
+from __future__ import annotations
+
+import json
+import os
+
+import torch
+from safetensors.torch import save_file
+
+from ..config.registry import architecture_of
+
+
+def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std: float = 0.02) -> dict:
+    from ..models.decoder import Decoder
+    model = Decoder(architecture_of(config).build(config))
+    gen = torch.Generator(device="cpu").manual_seed(int(seed))
+    out = {}
+    for _, spec in model.param_specs():
+        for s in spec.sources:
+            if s.name in out:
+                continue
+            if spec.integer:
+                raise NotImplementedError("random integer tables")
+            t = torch.randn(s.shape, generator=gen, dtype=torch.float32) * std
+            if len(s.shape) == 1:
+                t = t + 1.0
+            out[s.name] = t.to(dtype).contiguous()
+    return out
+
+
+def write_random_model(config, seed: int, folder: str, dtype: torch.dtype = torch.bfloat16, std: float = 0.02) -> str:
+    os.makedirs(folder, exist_ok=True)
+    d = config.to_dict()
+    d["torch_dtype"] = str(dtype).replace("torch.", "")
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(d, f, indent=1)
+    save_file(random_tensors(config, seed, dtype, std), os.path.join(folder, "model.safetensors"))
+    return folder
