@@ -42,8 +42,9 @@ class CacheManager:
         self.pools = [IdPool(g.num_pages, 1, "page") for g in self.groups]
         self.slots = IdPool(num_state_slots, 1, "state slot")
         self.live: dict[object, RequestCache] = {}
-        self.released_log: list = []     # (group, page) in release order, for poisoning / tests
+        self.released_log: list = []     # (group, page) in release order, kept when keep_log is set
         self.keep_log = False
+        self.on_release = None           # callable(group, pages), called as pages go back (debugging)
 
     # ----------------------------------------------------------- lifecycle
     def can_open(self) -> bool:
@@ -75,6 +76,8 @@ class CacheManager:
         self.pools[g].give_back(pages)
         if self.keep_log:
             self.released_log.extend((g, p) for p in pages)
+        if self.on_release is not None and pages:
+            self.on_release(g, pages)
 
     # ------------------------------------------------------------ reserving
     def pages_needed(self, rc: RequestCache, num_computed: int, n: int) -> list[int]:

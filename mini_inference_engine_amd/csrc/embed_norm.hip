@@ -1,0 +1,111 @@
+// Token embedding into the 32-bit residual stream, and the residual add fused with RMSNorm.
+//
+// embedding:    stream[t, :] = float(table[ids[t], :])
+// add_rmsnorm:  r = stream[row] (+ float(x[row]));  stream[row] = r (unless rows are gathered);
+//               y[row] = r * (1 / sqrt(mean(r^2) + eps)) * weight, rounded once to y's type.
+// One workgroup per row; the row's sum of squares is reduced in an order that depends only on
+// the row width, so a token's result does not depend on what else is in the batch.
+#include "common.hpp"
+
+template <typename TT>
+__global__ void embedding_kernel(const int* __restrict__ ids, const TT* __restrict__ table, float* __restrict__ out,
+                                 int width, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // ids are validated on the host; never read outside
+  const TT* src = table + (size_t)id * width;
+  float* dst = out + (size_t)t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float(src[i]);
+}
+
+#define NORM_THREADS 256
+#define NORM_CACHE 16
+
+template <typename TX, typename TW, typename TY>
+__global__ void __launch_bounds__(NORM_THREADS)
+add_rmsnorm_kernel(const TX* __restrict__ x, float* __restrict__ stream, const TW* __restrict__ weight,
+                   TY* __restrict__ y, const int* __restrict__ rows, int width, float eps) {
+  __shared__ float scratch[16];
+  const int out_row = blockIdx.x;
+  const int row = rows ? rows[out_row] : out_row;
+  float* sr = stream + (size_t)row * width;
+  const TX* xr = x ? x + (size_t)row * width : nullptr;
+  float cache[NORM_CACHE];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NORM_CACHE; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    float r = 0.f;
+    if (i < width) {
+      r = sr[i];
+      if (xr) r += to_float(xr[i]);
+      if (xr && !rows) sr[i] = r;
+    }
+    cache[k] = r;
+    ss += r * r;
+  }
+  for (int i = threadIdx.x + NORM_CACHE * NORM_THREADS; i < width; i += NORM_THREADS) {
+    float r = sr[i];
+    if (xr) r += to_float(xr[i]);
+    if (xr && !rows) sr[i] = r;
+    ss += r * r;
+  }
+  const float total = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(total / (float)width + eps);
+  TY* yr = y + (size_t)out_row * width;
+#pragma unroll
+  for (int k = 0; k < NORM_CACHE; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    if (i < width) yr[i] = from_float<TY>(cache[k] * rstd * to_float(weight[i]));
+  }
+  for (int i = threadIdx.x + NORM_CACHE * NORM_THREADS; i < width; i += NORM_THREADS) {
+    float r = sr[i];
+    if (xr && rows) r += to_float(xr[i]);   // gathered rows were not written back
+    yr[i] = from_float<TY>(r * rstd * to_float(weight[i]));
+  }
+}
+
+MIE_EXPORT const char* embed_norm_last_error() { return g_mie_error; }
+
+MIE_EXPORT int mie_embedding(const int* ids, const void* table, int table_dtype, float* out, int tokens, int width,
+                             int vocab, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (width <= 0 || vocab <= 0) MIE_FAIL("embedding: width %d, vocab %d", width, vocab);
+  dim3 grid(tokens), block(256);
+  if (table_dtype == MIE_F32)
+    hipLaunchKernelGGL(embedding_kernel<float>, grid, block, 0, stream, ids, (const float*)table, out, width, vocab);
+  else if (table_dtype == MIE_BF16)
+    hipLaunchKernelGGL(embedding_kernel<bf16>, grid, block, 0, stream, ids, (const bf16*)table, out, width, vocab);
+  else
+    MIE_FAIL("embedding: table dtype code %d", table_dtype);
+  MIE_CHECK_LAUNCH("embedding");
+  return 0;
+}
+
+template <typename TX, typename TW>
+static int launch_norm(const void* x, float* stream, const void* w, void* y, int y_dtype, const int* rows, int n_rows,
+                       int width, float eps, hipStream_t s) {
+  dim3 grid(n_rows), block(NORM_THREADS);
+  if (y_dtype == MIE_F32)
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TX, TW, float>), grid, block, 0, s, (const TX*)x, stream, (const TW*)w,
+                       (float*)y, rows, width, eps);
+  else if (y_dtype == MIE_BF16)
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TX, TW, bf16>), grid, block, 0, s, (const TX*)x, stream, (const TW*)w,
+                       (bf16*)y, rows, width, eps);
+  else
+    MIE_FAIL("add_rmsnorm: output dtype code %d", y_dtype);
+  MIE_CHECK_LAUNCH("add_rmsnorm");
+  return 0;
+}
+
+// x may be null (nothing to add).  rows may be null (all n_rows rows, stream updated in place).
+MIE_EXPORT int mie_add_rmsnorm(const void* x, int x_dtype, float* stream, const void* weight, int w_dtype, void* y,
+                               int y_dtype, const int* rows, int n_rows, int width, float eps, hipStream_t s) {
+  if (n_rows <= 0) return 0;
+  if (width <= 0) MIE_FAIL("add_rmsnorm: width %d", width);
+  if (x_dtype == MIE_F32 && w_dtype == MIE_F32) return launch_norm<float, float>(x, stream, weight, y, y_dtype, rows, n_rows, width, eps, s);
+  if (x_dtype == MIE_F32 && w_dtype == MIE_BF16) return launch_norm<float, bf16>(x, stream, weight, y, y_dtype, rows, n_rows, width, eps, s);
+  if (x_dtype == MIE_BF16 && w_dtype == MIE_F32) return launch_norm<bf16, float>(x, stream, weight, y, y_dtype, rows, n_rows, width, eps, s);
+  if (x_dtype == MIE_BF16 && w_dtype == MIE_BF16) return launch_norm<bf16, bf16>(x, stream, weight, y, y_dtype, rows, n_rows, width, eps, s);
+  MIE_FAIL("add_rmsnorm: dtype codes x %d, weight %d", x_dtype, w_dtype);
+}

@@ -115,15 +115,16 @@ def order_rows(rows: Sequence[StepRow]) -> list[int]:
 
 
 def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad_rows_to: int = 0,
-               static_context: int = 0) -> StepContext:
+               static_context: int = 0, want_all: bool = False) -> StepContext:
     """Flatten ``rows`` into ``arena``.  ``pad_rows_to`` adds scratch rows (one token at
-    position 0, page 0, slot 0) up to a captured batch size; their logits are not wanted."""
+    position 0, page 0, slot 0) up to a captured batch size.  ``want_all`` asks for the logits
+    of every token in flat order (what a captured step produces) instead of the rows' wants."""
     order = order_rows(rows)
     n_rows = len(rows)
     lens = np.fromiter((len(rows[i].tokens) for i in order), dtype=np.int64, count=n_rows)
-    if n_rows == 0 or (lens <= 0).any():
-        raise ValueError("a step needs at least one row and every row at least one token")
     total_rows = max(n_rows, pad_rows_to)
+    if total_rows == 0 or (lens <= 0).any():
+        raise ValueError("a step needs at least one row and every row at least one token")
     pad = total_rows - n_rows
     T = int(lens.sum()) + pad
     if T > arena.max_tokens or total_rows > arena.max_rows:
@@ -142,7 +143,7 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
     token_row = np.repeat(np.arange(total_rows), row_len)
     positions = np.arange(T) - row_start[token_row] + row_pos[token_row]
     ctx = row_pos + row_len
-    blocks_needed = int(-(-ctx.max() // page_size))
+    blocks_needed = int(-(-int(ctx.max()) // page_size))
     if blocks_needed > arena.max_blocks:
         raise ValueError(f"a row needs {blocks_needed} pages; the arena holds {arena.max_blocks} per row")
 
@@ -165,8 +166,8 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
     arena.host_view("row_context")[:total_rows] = ctx
 
     # wanted logits, in the caller's order of rows and of ``want``
-    wanted = []
-    for i, r in enumerate(rows):
+    wanted = list(range(T)) if want_all else []
+    for i, r in enumerate(rows if not want_all else ()):
         base = row_start[new_row_of[i]]
         for w in r.want:
             if not 0 <= w < len(r.tokens):

@@ -1,0 +1,57 @@
+"""Captured decode steps: one hipGraph per batch-size bucket.
+
+A step of single-token rows is launch-bound when run kernel by kernel.  As in the
+reference (inference_engine/engine.py:76-120), the whole forward of such a step is
+captured once per bucket on static buffers (the step arena) and replayed; a batch is
+padded to its bucket with scratch rows that read and write page 0.  Everything a
+kernel needs that changes from step to step (token ids, positions, block tables,
+slots) is read from the arena on the device, so a replay needs only the arena's
+upload.  No memset node is recorded: buffers are cleared by kernels.
+"""
+from __future__ import annotations
+
+import time
+
+import torch
+
+
+class DecodeGraphs:
+    def __init__(self, runner, cfg, verbose: bool = True):
+        self.runner = runner
+        self.sizes = sorted(b for b in set(cfg.graph_batch_sizes) if b <= cfg.max_num_seqs
+                            and b <= cfg.max_num_batched_tokens)
+        self.graphs = {}
+        self.static_context = runner.max_model_len
+        if not self.sizes:
+            return
+        t0 = time.perf_counter()
+        pool = None
+        for bs in reversed(self.sizes):                 # largest first: smaller ones reuse its pool
+            step = runner.build([], pad_rows_to=bs, static_context=self.static_context, want_all=True)
+            runner.model.forward(step)                  # loads libraries, warms the allocator
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, pool=pool):
+                logits = runner.model.forward(step)
+            pool = g.pool()
+            self.graphs[bs] = (g, logits)
+        torch.cuda.synchronize()
+        if verbose:
+            print(f"[mini_inference_engine_amd] captured {len(self.sizes)} decode graphs "
+                  f"(batch <= {self.sizes[-1]}) in {time.perf_counter() - t0:.1f} s", flush=True)
+
+    def fits(self, rows: int) -> bool:
+        return bool(self.sizes) and rows <= self.sizes[-1]
+
+    def run(self, rows) -> torch.Tensor | None:
+        """``rows``: single-token StepRows.  Logits of the rows that want them, in order."""
+        bs = next(s for s in self.sizes if s >= len(rows))
+        picked = [i for i, r in enumerate(rows) if len(r.want)]
+        self.runner.build(rows, pad_rows_to=bs, static_context=self.static_context, want_all=True)
+        g, logits = self.graphs[bs]
+        g.replay()
+        if not picked:
+            return None
+        if len(picked) == len(rows):
+            return logits[:len(rows)]
+        return logits[torch.tensor(picked, device=logits.device)]

@@ -1,0 +1,164 @@
+"""The offline entry point: add requests, step until done.
+
+Surface as the reference's (inference_engine/engine.py:17-24,35-37,123,181,232):
+``LLMEngine(model, engine_config, dtype, load_tokenizer, verbose)``,
+``add_request``, ``step`` (returns the requests that finished), ``generate``,
+``RequestOutput``; attributes ``scheduler``, ``cfg``, ``model_cfg``,
+``num_steps``, ``num_graph_steps``.  ``model`` is a folder (config.json and
+safetensors); prompts are lists of token ids (strings only when a tokenizer
+was loaded).
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, replace
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..sampling import Sampler, SamplingParams
+from .batch import StepRow
+from .runner import ModelRunner, parse_dtype
+from .scheduler import Scheduler
+from .sequence import Sequence
+
+
+@dataclass
+class RequestOutput:
+    seq_id: int
+    prompt_len: int
+    output_ids: list
+    text: str | None
+    ttft: float | None          # seconds from arrival to the first generated token
+    latency: float | None       # seconds from arrival to the end
+
+
+class LLMEngine:
+    def __init__(self, model, engine_config: EngineConfig | None = None, dtype=torch.bfloat16,
+                 load_tokenizer: bool = False, verbose: bool = True, *, device="cuda", backend=None, weights=None):
+        self.cfg = engine_config or EngineConfig()
+        self.verbose = verbose
+        self.dtype = parse_dtype(dtype)
+        cfg = self.cfg
+        self.runner = ModelRunner(
+            model, dtype=self.dtype, device=device, backend=backend, page_size=cfg.block_size,
+            num_pages=cfg.num_blocks, memory_fraction=cfg.kv_cache_memory_fraction,
+            reserve_bytes=cfg.activation_reserve_bytes, max_step_tokens=cfg.max_num_batched_tokens,
+            max_rows=cfg.max_num_seqs, max_model_len=cfg.max_model_len, num_state_slots=cfg.num_state_slots,
+            weights=weights)
+        self.model_cfg = self.runner.model_cfg
+        self.cfg.max_model_len = self.runner.max_model_len
+        self.cache = self.runner.cache
+        self.allocator = self.cache            # the name the reference's callers use
+        if cfg.poison_freed_pages:
+            self.cache.on_release = self.runner.storage.poison_pages
+        self.scheduler = Scheduler(self.cfg, self.cache)
+        self.sampler = Sampler(self.runner.ops, self.runner.device, cfg.max_num_seqs)
+        self.eos_token_id = self.runner.model.spec.eos_token_id
+        if verbose:
+            print(f"[mini_inference_engine_amd] cache: {self.runner.num_pages} pages x {cfg.block_size} tokens "
+                  f"({self.runner.storage.num_bytes() / 2**30:.2f} GiB), weights "
+                  f"{self.runner.model.weight_bytes() / 2**30:.2f} GiB, dtype {self.dtype}", flush=True)
+        self.tokenizer = None
+        if load_tokenizer and isinstance(model, str):
+            from transformers import AutoTokenizer      # text in and out only; never on the token path
+            self.tokenizer = AutoTokenizer.from_pretrained(model)
+        self.graphs = None
+        if cfg.use_hip_graphs and self.runner.device.type == "cuda":
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(self.runner, cfg, verbose=verbose)
+        self.num_steps = 0
+        self.num_graph_steps = 0
+        self._num_requests = 0
+
+    # ---------------------------------------------------------------- requests
+    def add_request(self, prompt, params: SamplingParams | None = None) -> Sequence:
+        if isinstance(prompt, str):
+            if self.tokenizer is None:
+                raise ValueError("a text prompt needs a tokenizer (load_tokenizer=True); pass token ids instead")
+            ids = self.tokenizer.encode(prompt)
+        else:
+            ids = list(prompt)
+        params = params or SamplingParams()
+        if len(ids) > self.cfg.max_model_len:
+            raise ValueError(f"prompt of {len(ids)} tokens exceeds max_model_len {self.cfg.max_model_len}")
+        vocab = self.runner.vocab_size
+        bad = [t for t in ids if not 0 <= t < vocab]
+        if bad:
+            raise ValueError(f"token ids outside the vocabulary of {vocab}: {bad[:5]}")
+        if len(ids) + params.max_tokens > self.cfg.max_model_len:
+            params = replace(params, max_tokens=self.cfg.max_model_len - len(ids))
+        seq = Sequence(ids, params)
+        if params.seed is None:
+            seq.seed = (self.cfg.seed << 32) ^ self._num_requests
+        self._num_requests += 1
+        self.scheduler.add(seq)
+        return seq
+
+    # ------------------------------------------------------------------- step
+    def step(self) -> list[Sequence]:
+        """One scheduling + forward + sampling step.  Returns the requests that finished."""
+        batch = self.scheduler.schedule()
+        if not batch:
+            return []
+        rows, sample_seqs = [], []
+        for seq, n in batch:
+            nc = seq.num_computed
+            last = nc + n == seq.num_tokens
+            rows.append(StepRow(seq.cache, seq.token_ids[nc:nc + n], nc, [n - 1] if last else []))
+            if last:
+                sample_seqs.append(seq)
+
+        pure_decode = all(n == 1 for _, n in batch)
+        if pure_decode and self.graphs is not None and self.graphs.fits(len(rows)):
+            logits = self.graphs.run(rows)
+            self.num_graph_steps += 1
+        else:
+            logits = self.runner.forward_step(rows)
+
+        new_tokens = []
+        if sample_seqs:
+            new_tokens = self.sampler.sample(
+                logits, [s.params.temperature for s in sample_seqs], [s.seed for s in sample_seqs],
+                [s.num_output_tokens for s in sample_seqs])
+
+        self.num_steps += 1
+        for seq, n in batch:
+            self.scheduler.advance(seq, n)
+        now = time.perf_counter()
+        finished = []
+        for seq, tok in zip(sample_seqs, new_tokens):
+            seq.token_ids.append(tok)
+            if seq.first_token_time is None:
+                seq.first_token_time = now
+            done = (seq.num_output_tokens >= seq.params.max_tokens
+                    or seq.num_tokens >= self.cfg.max_model_len
+                    or (tok == self.eos_token_id and not seq.params.ignore_eos))
+            if done:
+                seq.finish_time = now
+                self.scheduler.finish(seq)
+                finished.append(seq)
+        return finished
+
+    # --------------------------------------------------------------- offline
+    def generate(self, prompts, params: SamplingParams | list | None = None, decode_text: bool = True
+                 ) -> list[RequestOutput]:
+        if not isinstance(params, list):
+            params = [params or SamplingParams()] * len(prompts)
+        if len(params) != len(prompts):
+            raise ValueError(f"{len(prompts)} prompts but {len(params)} sampling params")
+        seqs = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        done_early = [s for s in seqs if s.params.max_tokens == 0]
+        for s in done_early:                     # nothing to generate: never scheduled
+            self.scheduler.waiting.remove(s)
+            s.finish_time = s.first_token_time = time.perf_counter()
+        while self.scheduler.has_work():
+            self.step()
+        outs = []
+        for s in seqs:
+            text = None
+            if decode_text and self.tokenizer is not None:
+                text = self.tokenizer.decode(s.output_ids, skip_special_tokens=True)
+            outs.append(RequestOutput(s.seq_id, s.prompt_len, s.output_ids, text,
+                                      s.first_token_time - s.arrival_time, s.finish_time - s.arrival_time))
+        return outs

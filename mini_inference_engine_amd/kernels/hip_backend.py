@@ -1,0 +1,263 @@
+"""The kernels the engine computes with: hand-written HIP for gfx950, called through ctypes.
+
+Every wrapper checks on the host that operand shapes, dtypes and strides are what
+its kernel and grid assume before anything is launched, launches on torch's
+current stream, and raises with the library's message on a refusal.  Matrix
+products of the bfloat16 path with many rows go to the library GEMM behind
+torch (hipBLASLt), as the reference's go to cuBLAS (inference_engine/model.py:172-185);
+everything else, and every product of the float32 path, is a kernel of this
+package.  There is no CPU path and no fallback: a missing library is an error.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+
+import torch
+
+from . import library
+from .api import KernelBackend
+
+F32, BF16 = 0, 1
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise TypeError(f"kernels take float32 or bfloat16, not {dtype}")
+
+
+def _ptr(t) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _rows_ok(t: torch.Tensor, what: str) -> None:
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"{what}: expected a 2-d tensor with unit inner stride, got shape {tuple(t.shape)} "
+                         f"strides {t.stride()}")
+
+
+class HipBackend(KernelBackend):
+    name = "hip-gfx950"
+
+    # rows at or above which the bfloat16 products go to the library GEMM
+    LIBRARY_GEMM_ROWS = 1
+
+    def __init__(self, act_dtype: torch.dtype, device="cuda"):
+        self.act_dtype = act_dtype
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError("the HIP kernels run on the GPU only; there is no CPU path")
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU visible to torch: the engine needs an MI355X (gfx950)")
+        self._libs = {}
+        self.true_fp32 = act_dtype == torch.float32
+
+    # ------------------------------------------------------------ plumbing
+    def lib(self, module: str, defines: tuple = ()):
+        key = (module, defines)
+        if key not in self._libs:
+            lib = library.load(module, defines)
+            self._declare(module, lib)
+            self._libs[key] = lib
+        return self._libs[key]
+
+    @staticmethod
+    def _declare(module: str, lib) -> None:
+        sig = {
+            "embed_norm": {
+                "mie_embedding": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+                "mie_add_rmsnorm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                                    c_int, c_float, c_void_p],
+            },
+            "rope_kv": {
+                "mie_rotary_kv_store": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                        c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+            },
+            "gemm": {
+                "mie_gemm_nt": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_void_p,
+                                c_int, c_int, c_int, c_void_p],
+                "mie_silu_mul": [c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
+            },
+            "attention": {
+                "mie_paged_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                        c_void_p],
+            },
+            "sampling": {
+                "mie_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+            },
+        }.get(module, {})
+        for name, argtypes in sig.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = c_int
+
+    def _stream(self) -> c_void_p:
+        return c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _on_device(self, *tensors) -> None:
+        for t in tensors:
+            if t is not None and t.device.type != "cuda":
+                raise ValueError(f"tensor on {t.device}; the kernels take GPU tensors only")
+
+    # ----------------------------------------------------------------- ops
+    def embedding(self, ids, table):
+        self._on_device(ids, table)
+        if ids.dtype != torch.int32 or ids.dim() != 1 or not ids.is_contiguous():
+            raise ValueError("embedding: ids must be contiguous int32 [T]")
+        if table.dim() != 2 or not table.is_contiguous():
+            raise ValueError("embedding: table must be contiguous [vocab, width]")
+        T, (V, W) = ids.shape[0], table.shape
+        out = torch.empty((T, W), dtype=torch.float32, device=table.device)
+        lib = self.lib("embed_norm")
+        library.check(lib, lib.mie_embedding(_ptr(ids), _ptr(table), _code(table.dtype), _ptr(out), T, W, V,
+                                             self._stream()))
+        return out
+
+    def add_rmsnorm(self, x, residual, weight, eps, out_dtype=None, rows=None):
+        self._on_device(x, residual, weight, rows)
+        out_dtype = out_dtype or self.act_dtype
+        if residual.dtype != torch.float32 or residual.dim() != 2 or not residual.is_contiguous():
+            raise ValueError("add_rmsnorm: the residual stream must be contiguous float32 [T, width]")
+        T, W = residual.shape
+        if x is not None and (tuple(x.shape) != (T, W) or not x.is_contiguous()):
+            raise ValueError(f"add_rmsnorm: x {tuple(x.shape)} does not match the stream {(T, W)}")
+        if tuple(weight.shape) != (W,) or not weight.is_contiguous():
+            raise ValueError(f"add_rmsnorm: weight {tuple(weight.shape)} for width {W}")
+        n = T
+        if rows is not None:
+            if rows.dtype != torch.int32 or rows.dim() != 1 or not rows.is_contiguous():
+                raise ValueError("add_rmsnorm: rows must be contiguous int32")
+            n = rows.shape[0]
+        y = torch.empty((n, W), dtype=out_dtype, device=residual.device)
+        lib = self.lib("embed_norm")
+        library.check(lib, lib.mie_add_rmsnorm(
+            _ptr(x), _code(x.dtype) if x is not None else F32, _ptr(residual), _ptr(weight), _code(weight.dtype),
+            _ptr(y), _code(out_dtype), _ptr(rows), n, W, float(eps), self._stream()))
+        return y
+
+    def _gemm(self, x, w, bias, out_dtype):
+        M, K = x.shape
+        N = w.shape[0]
+        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        if bias is not None:
+            bias = bias.float().contiguous()
+        lib = self.lib("gemm")
+        library.check(lib, lib.mie_gemm_nt(_ptr(x), _code(x.dtype), x.stride(0), _ptr(w), _code(w.dtype), w.stride(0),
+                                           _ptr(y), _code(out_dtype), y.stride(0), _ptr(bias), M, N, K,
+                                           self._stream()))
+        return y
+
+    def linear(self, x, w, bias=None, out_dtype=None):
+        self._on_device(x, w, bias)
+        _rows_ok(x, "linear: x")
+        _rows_ok(w, "linear: w")
+        if x.shape[1] != w.shape[1]:
+            raise ValueError(f"linear: x {tuple(x.shape)} against w {tuple(w.shape)}")
+        out_dtype = out_dtype or self.act_dtype
+        if (not self.true_fp32 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+                and x.shape[0] >= self.LIBRARY_GEMM_ROWS):
+            # library matrix product, 32-bit accumulation, as the reference's F.linear
+            y = torch.nn.functional.linear(x, w, None if bias is None else bias.to(torch.bfloat16))
+            return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
+        return self._gemm(x, w, bias, out_dtype)
+
+    def silu_mul(self, gu, intermediate):
+        _rows_ok(gu, "silu_mul: gu")
+        if gu.shape[1] != 2 * intermediate:
+            raise ValueError(f"silu_mul: {gu.shape[1]} columns for intermediate {intermediate}")
+        out = torch.empty((gu.shape[0], intermediate), dtype=gu.dtype, device=gu.device)
+        lib = self.lib("gemm")
+        library.check(lib, lib.mie_silu_mul(_ptr(gu), gu.stride(0), _ptr(out), out.stride(0), _code(gu.dtype),
+                                            gu.shape[0], intermediate, self._stream()))
+        return out
+
+    def linear_silu_mul(self, x, w_gate_up, intermediate):
+        if w_gate_up.shape[0] != 2 * intermediate:
+            raise ValueError(f"linear_silu_mul: weight of {w_gate_up.shape[0]} rows for intermediate {intermediate}")
+        return self.silu_mul(self.linear(x, w_gate_up), intermediate)
+
+    def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
+                        k_cache, v_cache, slot_mapping):
+        self._on_device(qkv, positions, cos, sin, k_cache, v_cache, slot_mapping)
+        _rows_ok(qkv, "rotary_kv_store: qkv")
+        T = qkv.shape[0]
+        Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
+        if qkv.shape[1] != (Hq + 2 * Hkv) * D:
+            raise ValueError(f"rotary_kv_store: qkv has {qkv.shape[1]} columns, expected {(Hq + 2 * Hkv) * D}")
+        page = 0
+        if rotary_dim:
+            half = rotary_dim // 2
+            for name, t in (("cos", cos), ("sin", sin)):
+                if t is None or t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != half or not t.is_contiguous():
+                    raise ValueError(f"rotary_kv_store: {name} must be contiguous float32 [positions, {half}]")
+            if positions.dtype != torch.int32 or positions.shape[0] != T or not positions.is_contiguous():
+                raise ValueError("rotary_kv_store: positions must be contiguous int32 [T]")
+        if Hkv:
+            page = k_cache.shape[2]
+            want = (k_cache.shape[0], Hkv, page, D)
+            for name, t in (("k_cache", k_cache), ("v_cache", v_cache)):
+                if tuple(t.shape) != want or t.dtype != qkv.dtype or not t.is_contiguous():
+                    raise ValueError(f"rotary_kv_store: {name} {tuple(t.shape)} {t.dtype}, expected {want} {qkv.dtype}")
+            if slot_mapping.dtype != torch.int32 or slot_mapping.shape[0] != T or not slot_mapping.is_contiguous():
+                raise ValueError("rotary_kv_store: slot_mapping must be contiguous int32 [T]")
+        lib = self.lib("rope_kv")
+        library.check(lib, lib.mie_rotary_kv_store(
+            _ptr(qkv), _code(qkv.dtype), qkv.stride(0), _ptr(positions), _ptr(cos), _ptr(sin), rotary_dim, Hq, Hkv, D,
+            _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), page, T, self._stream()))
+
+    def _check_attention(self, qkv, Hq, Hkv, D, k_cache, v_cache, group, step):
+        _rows_ok(qkv, "paged_attention: qkv")
+        T = qkv.shape[0]
+        if qkv.shape[1] < Hq * D:
+            raise ValueError(f"paged_attention: qkv has {qkv.shape[1]} columns, fewer than {Hq * D}")
+        pages, hk, page, d = k_cache.shape
+        if (hk, d) != (Hkv, D) or tuple(v_cache.shape) != tuple(k_cache.shape):
+            raise ValueError(f"paged_attention: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for "
+                             f"{Hkv} kv heads of {D}")
+        if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype or not (k_cache.is_contiguous() and
+                                                                            v_cache.is_contiguous()):
+            raise ValueError("paged_attention: caches must be contiguous and of the activation dtype")
+        bt = group.block_tables
+        if bt.dtype != torch.int32 or bt.dim() != 2 or bt.stride(1) != 1 or bt.stride(0) != bt.shape[1]:
+            raise ValueError("paged_attention: block tables must be contiguous int32 [rows, max_blocks]")
+        if bt.shape[0] < step.num_rows:
+            raise ValueError(f"paged_attention: {bt.shape[0]} block-table rows for {step.num_rows} rows")
+        for name, t in (("token_row", step.token_row), ("positions", step.positions)):
+            if t.dtype != torch.int32 or t.shape[0] != T or not t.is_contiguous():
+                raise ValueError(f"paged_attention: {name} must be contiguous int32 [T]")
+        if step.max_context > bt.shape[1] * page:
+            raise ValueError(f"paged_attention: context {step.max_context} exceeds the block tables "
+                             f"({bt.shape[1]} pages of {page})")
+        return T, page, bt
+
+    def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
+                        window):
+        self._on_device(qkv, k_cache, v_cache)
+        Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
+        T, page, bt = self._check_attention(qkv, Hq, Hkv, D, k_cache, v_cache, group, step)
+        out = torch.empty((T, Hq * D), dtype=qkv.dtype, device=qkv.device)
+        lib = self.lib("attention")
+        library.check(lib, lib.mie_paged_attention(
+            _ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _code(qkv.dtype), _ptr(bt),
+            bt.shape[1], _ptr(step.token_row), _ptr(step.positions), T, Hq, Hkv, D, page, float(scale),
+            int(window or 0), self._stream()))
+        return out
+
+    def sample(self, logits, temperatures, seeds, counters):
+        self._on_device(logits, temperatures, seeds, counters)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+            raise ValueError("sample: logits must be float32 [rows, vocab] with unit inner stride")
+        R, V = logits.shape
+        if (temperatures.dtype, seeds.dtype, counters.dtype) != (torch.float32, torch.int64, torch.int32):
+            raise ValueError("sample: temperatures float32, seeds int64, counters int32")
+        if not (temperatures.shape[0] == seeds.shape[0] == counters.shape[0] == R):
+            raise ValueError("sample: one temperature, seed and counter per row")
+        out = torch.empty(R, dtype=torch.int32, device=logits.device)
+        lib = self.lib("sampling")
+        library.check(lib, lib.mie_sample(_ptr(logits), logits.stride(0), _ptr(temperatures), _ptr(seeds),
+                                          _ptr(counters), _ptr(out), R, V, self._stream()))
+        return out

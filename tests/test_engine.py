@@ -1,0 +1,181 @@
+"""Generation through the entry point (LLMEngine.generate) against the plain implementation.
+
+Configuration A: prompts of 5/17/33 tokens, 8 greedy tokens each.  Configuration B: prompts of
+1/9/40/70 tokens, 12 tokens at temperature 0.8 from seeded streams, token budget 32 so that
+prompts are cut into portions that share steps with decoding requests.  Without a GPU the
+engine runs on the kernel references (host logic only); with one, on the HIP kernels.
+
+A sampled or greedy token is accepted if, on the plain implementation's logits for the same
+prefix, its (perturbed) score is within ``slack`` of the best: two implementations that round
+differently may break a near-tie differently, and nothing else may differ.
+"""
+import pytest
+import torch
+
+import plain_llama
+from torch_backend import TorchBackend, ref_perturbed
+
+from mini_inference_engine_amd import LLMEngine, SamplingParams
+from mini_inference_engine_amd.config import EngineConfig
+
+
+def check_outputs(m, prompts, outs, params, slack_rel, weights_key="weights"):
+    for prompt, out, sp in zip(prompts, outs, params):
+        ids = list(prompt)
+        assert len(out.output_ids) == sp.max_tokens
+        for i, tok in enumerate(out.output_ids):
+            logits = plain_llama.forward(m["cfg"], m[weights_key], ids)[-1]
+            z = ref_perturbed(logits, sp.temperature, sp.seed if sp.seed is not None else 0, i)
+            slack = slack_rel * float(logits.abs().max()) / max(sp.temperature, 1e-9 if sp.temperature else 1.0)
+            assert float(z.max() - z[tok]) <= slack, \
+                f"request of {len(prompt)} tokens, output {i}: token {tok}, plain chooses {int(z.argmax())}"
+            ids.append(tok)
+
+
+def prompts_for(m, lengths, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, m["cfg"]["vocab_size"], (n,), generator=g).tolist() for n in lengths]
+
+
+def engine(m, device, dtype, **cfg):
+    if device == "cpu":
+        return LLMEngine(m["config"], EngineConfig(**cfg), dtype=dtype, verbose=False, device="cpu",
+                         backend=TorchBackend(torch.float32), weights=m["weights"])
+    folder = m["folder_f32"] if dtype == "float32" else m["folder_bf16"]
+    return LLMEngine(folder, EngineConfig(**cfg), dtype=dtype, verbose=False)
+
+
+def run_a(m, device, dtype, slack, **cfg):
+    prompts = prompts_for(m, [5, 17, 33])
+    eng = engine(m, device, dtype, num_blocks=16, max_num_seqs=4, **cfg)
+    sp = SamplingParams(max_tokens=8, ignore_eos=True)
+    outs = eng.generate(prompts, sp)
+    check_outputs(m, prompts, outs, [sp] * 3, slack, "weights" if dtype == "float32" else "weights_bf16")
+    eng.cache.check()
+    assert not eng.cache.live and eng.cache.num_free(0) == 15
+    return eng
+
+
+def run_b(m, device, dtype, slack, **cfg):
+    prompts = prompts_for(m, [1, 9, 40, 70], seed=1)
+    eng = engine(m, device, dtype, num_blocks=24, max_num_seqs=4, max_num_batched_tokens=32, **cfg)
+    params = [SamplingParams(max_tokens=12, temperature=0.8, ignore_eos=True, seed=100 + i) for i in range(4)]
+    outs = eng.generate(prompts, params)
+    check_outputs(m, prompts, outs, params, slack, "weights" if dtype == "float32" else "weights_bf16")
+    eng.cache.check()
+    return eng
+
+
+def test_generate_a_host(tiny_models):
+    run_a(tiny_models["A"], "cpu", "float32", 1e-6)
+
+
+def test_generate_b_host(tiny_models):
+    eng = run_b(tiny_models["B"], "cpu", "float32", 1e-6)
+    assert eng.num_steps > 12, "budget 32 must cut the prompts into portions"
+
+
+def test_generate_under_preemption_host(tiny_models):
+    """So few pages that running requests are preempted and recomputed; tokens must not change."""
+    m = tiny_models["A"]
+    prompts = prompts_for(m, [30, 28, 33, 20], seed=2)
+    sp = SamplingParams(max_tokens=24, ignore_eos=True)
+    roomy = engine(m, "cpu", "float32", num_blocks=40, max_num_seqs=4).generate(prompts, sp)
+    tight_engine = engine(m, "cpu", "float32", num_blocks=10, max_num_seqs=4)
+    tight = tight_engine.generate(prompts, sp)
+    assert tight_engine.scheduler.num_preemptions > 0, "the preemption path was not exercised"
+    assert [o.output_ids for o in tight] == [o.output_ids for o in roomy]
+    tight_engine.cache.check()
+
+
+def test_same_seed_same_tokens_whatever_the_batch(tiny_models):
+    m = tiny_models["B"]
+    prompts = prompts_for(m, [9, 40, 21], seed=4)
+    params = [SamplingParams(max_tokens=10, temperature=1.0, ignore_eos=True, seed=7 + i) for i in range(3)]
+    together = engine(m, "cpu", "float32", num_blocks=30, max_num_seqs=4, max_num_batched_tokens=16).generate(prompts, params)
+    for p, sp, o in zip(prompts, params, together):
+        alone = engine(m, "cpu", "float32", num_blocks=30, max_num_seqs=1).generate([p], sp)
+        assert alone[0].output_ids == o.output_ids
+
+
+def test_eos_stops_and_stays(tiny_models):
+    m = tiny_models["A"]
+    prompts = prompts_for(m, [12], seed=6)
+    free_run = engine(m, "cpu", "float32", num_blocks=16).generate(prompts, SamplingParams(max_tokens=20, ignore_eos=True))
+    toks = free_run[0].output_ids
+    eng = engine(m, "cpu", "float32", num_blocks=16)
+    eng.eos_token_id = toks[3]
+    out = eng.generate(prompts, SamplingParams(max_tokens=20))
+    stop = toks.index(toks[3])
+    assert out[0].output_ids == toks[:stop + 1], "generation ends with the stop token, which stays in the output"
+
+
+def test_entry_point_argument_errors(tiny_models):
+    m = tiny_models["A"]
+    eng = engine(m, "cpu", "float32", num_blocks=16)
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.add_request([1, 2, 999])
+    with pytest.raises(ValueError, match="tokenizer"):
+        eng.add_request("some text")
+    with pytest.raises(ValueError, match="max_model_len"):
+        eng.add_request([1] * 500)
+    seq = eng.add_request([1] * 100, SamplingParams(max_tokens=1000))
+    assert seq.params.max_tokens == 28, "max_tokens is clamped to max_model_len - prompt (engine.py:126-127 there)"
+
+
+# ------------------------------------------------------------------------ GPU
+@pytest.mark.gpu
+@pytest.mark.parametrize("graphs", [False, True])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_generate_a_gpu(tiny_models, dtype, graphs):
+    eng = run_a(tiny_models["A"], "cuda", dtype, 1e-5 if dtype == "float32" else 2e-2, use_hip_graphs=graphs)
+    assert (eng.num_graph_steps > 0) == graphs
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("graphs", [False, True])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_generate_b_gpu(tiny_models, dtype, graphs):
+    run_b(tiny_models["B"], "cuda", dtype, 1e-5 if dtype == "float32" else 2e-2, use_hip_graphs=graphs)
+
+
+@pytest.mark.gpu
+def test_graph_steps_equal_eager_steps(tiny_models):
+    """Captured decode steps replayed many times, with eager work in between, give the eager tokens."""
+    m = tiny_models["C"]
+    prompts = prompts_for(m, [3, 20, 41, 9, 15], seed=8)
+    sp = SamplingParams(max_tokens=40, ignore_eos=True)
+    eager = engine(m, "cuda", "float32", num_blocks=64, max_num_seqs=8, use_hip_graphs=False).generate(prompts, sp)
+    eng = engine(m, "cuda", "float32", num_blocks=64, max_num_seqs=8, use_hip_graphs=True, graph_batch_sizes=(1, 2, 4, 8))
+    captured = eng.generate(prompts, sp)
+    assert eng.num_graph_steps >= 30
+    assert [o.output_ids for o in captured] == [o.output_ids for o in eager]
+    again = eng.generate(prompts[:2], sp)          # the same graphs, replayed after other work
+    assert [o.output_ids for o in again] == [o.output_ids for o in eager[:2]]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_preemption_gpu(tiny_models, dtype):
+    m = tiny_models["A"]
+    prompts = prompts_for(m, [30, 28, 33, 20], seed=2)
+    sp = SamplingParams(max_tokens=24, ignore_eos=True)
+    eng = engine(m, "cuda", dtype, num_blocks=10, max_num_seqs=4, poison_freed_pages=True)
+    outs = eng.generate(prompts, sp)
+    assert eng.scheduler.num_preemptions > 0
+    check_outputs(m, prompts, outs, [sp] * 4, 1e-5 if dtype == "float32" else 2e-2,
+                  "weights" if dtype == "float32" else "weights_bf16")
+
+
+@pytest.mark.gpu
+def test_long_decoding_gpu(tiny_models):
+    """Several hundred decoded tokens: the last rows still match the plain implementation."""
+    m = tiny_models["C"]
+    prompt = prompts_for(m, [7], seed=3)[0]
+    sp = SamplingParams(max_tokens=400, ignore_eos=True)
+    out = engine(m, "cuda", "float32", num_blocks=40, max_num_seqs=2).generate([prompt], sp)[0]
+    ids = prompt + out.output_ids
+    logits = plain_llama.forward(m["cfg"], m["weights"], ids[:-1])
+    for i in (0, 1, 100, 250, 399):
+        row = logits[len(prompt) - 1 + i]
+        assert float(row.max() - row[out.output_ids[i]]) <= 1e-5

@@ -1,0 +1,346 @@
+"""Each HIP kernel alone against its plain reference (tests/torch_backend.py), at sizes
+other than the engine's tiny models: widths and vocabularies that are no power of two,
+head sizes in steps of 16, odd head counts and groups, scattered pages.
+
+Vectors taken from the reference's own kernel tests (tests/test_kernels.py:14-59 there):
+RMSNorm rows {1, 7, 256, 2048} x widths {2048, 4096, 896} at eps 1e-5 with the bfloat16
+tolerance atol 2e-2 / rtol 1e-2; decode attention at 32 query heads on 4 kv heads of 64,
+page 16, context lengths [1], [17], [1000], [2048], [5, 300, 1, 2047, 64, 65] and
+range(1, 200, 7), pages scattered by a random permutation, tolerance 2e-2.
+"""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+import torch_backend as ref
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from mini_inference_engine_amd.kernels.hip_backend import HipBackend
+    return {torch.float32: HipBackend(torch.float32, DEV), torch.bfloat16: HipBackend(torch.bfloat16, DEV)}
+
+
+def tol(dtype):
+    return dict(atol=2e-2, rtol=1e-2) if dtype == torch.bfloat16 else dict(atol=2e-6, rtol=1e-5)
+
+
+# ------------------------------------------------------------------ embedding
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding(ops, dtype):
+    torch.manual_seed(0)
+    table = torch.randn(331, 120, device=DEV).to(dtype)
+    ids = torch.randint(0, 331, (77,), device=DEV, dtype=torch.int32)
+    out = ops[dtype].embedding(ids, table)
+    assert out.dtype == torch.float32
+    assert torch.equal(out, ref.ref_embedding(ids, table))
+
+
+# -------------------------------------------------------------------- rmsnorm
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [2048, 4096, 896, 120, 5000])
+@pytest.mark.parametrize("rows", [1, 7, 256, 2048])
+def test_add_rmsnorm(ops, dtype, rows, width):
+    if rows == 2048 and width == 5000:
+        rows = 300
+    torch.manual_seed(rows * 7 + width)
+    x = torch.randn(rows, width, device=DEV).to(dtype)
+    stream = torch.randn(rows, width, device=DEV)
+    w = torch.randn(width, device=DEV).to(dtype)
+    s_ref = stream.clone()
+    y_ref = ref.ref_add_rmsnorm(x, s_ref, w, 1e-5, dtype)
+    s = stream.clone()
+    y = ops[dtype].add_rmsnorm(x, s, w, 1e-5)
+    assert torch.equal(s, s_ref), "the updated stream must be bit-equal to stream + x"
+    torch.testing.assert_close(y.float(), y_ref.float(), **tol(dtype))
+    # nothing to add: the stream is left as it is
+    s2 = stream.clone()
+    y2 = ops[dtype].add_rmsnorm(None, s2, w, 1e-5)
+    assert torch.equal(s2, stream)
+    torch.testing.assert_close(y2.float(), ref.ref_add_rmsnorm(None, stream.clone(), w, 1e-5, dtype).float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm_rows_and_weight_dtype(ops, dtype):
+    torch.manual_seed(3)
+    x = torch.randn(50, 4700, device=DEV).to(dtype)
+    stream = torch.randn(50, 4700, device=DEV)
+    w32 = torch.randn(4700, device=DEV)            # a weight stored in 32-bit stays so
+    rows = torch.tensor([49, 0, 7, 7, 13], device=DEV, dtype=torch.int32)
+    before = stream.clone()
+    y = ops[dtype].add_rmsnorm(x, stream, w32, 1e-6, out_dtype=dtype, rows=rows)
+    assert torch.equal(stream, before), "gathered rows must not touch the stream"
+    y_ref = ref.ref_add_rmsnorm(x, before.clone(), w32, 1e-6, dtype, rows)
+    torch.testing.assert_close(y.float(), y_ref.float(), **tol(dtype))
+
+
+def test_rmsnorm_against_library(ops):
+    """float32: equals torch's rms_norm; a wrong eps placement or a mean over the wrong size fails it."""
+    torch.manual_seed(4)
+    x = torch.randn(9, 300, device=DEV) * 1e-3      # small values: eps matters
+    w = torch.randn(300, device=DEV)
+    y = ops[torch.float32].add_rmsnorm(None, x.clone(), w, 1e-5)
+    torch.testing.assert_close(y, torch.nn.functional.rms_norm(x, (300,), w, 1e-5), atol=1e-6, rtol=1e-5)
+
+
+# ----------------------------------------------------------------------- gemm
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1, 64, 176), (7, 200, 331), (130, 96, 120), (65, 1030, 77), (300, 512, 640)])
+def test_linear(ops, dtype, shape):
+    M, K, N = shape
+    torch.manual_seed(M + N)
+    x = torch.randn(M, K, device=DEV).to(dtype)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(dtype)
+    y = ops[dtype].linear(x, w)
+    torch.testing.assert_close(y.float(), ref.ref_linear(x, w, None, dtype).float(), **tol(dtype))
+    y32 = ops[dtype].linear(x, w, out_dtype=torch.float32)
+    assert y32.dtype == torch.float32
+    torch.testing.assert_close(y32, ref.ref_linear(x, w, None, torch.float32), **tol(dtype))
+
+
+def test_linear_float32_is_batch_invariant(ops):
+    torch.manual_seed(1)
+    x = torch.randn(200, 333, device=DEV)
+    w = torch.randn(150, 333, device=DEV)
+    whole = ops[torch.float32].linear(x, w)
+    for a, b in ((0, 1), (63, 130), (199, 200), (17, 19)):
+        assert torch.equal(ops[torch.float32].linear(x[a:b].contiguous(), w), whole[a:b])
+
+
+def test_linear_mixed_storage(ops):
+    """A matrix stored in 32-bit beside bfloat16 activations: computed, not refused."""
+    torch.manual_seed(2)
+    x = torch.randn(9, 120, device=DEV).to(torch.bfloat16)
+    w = torch.randn(50, 120, device=DEV) / 11
+    y = ops[torch.bfloat16].linear(x, w)
+    assert y.dtype == torch.bfloat16
+    torch.testing.assert_close(y.float(), ref.ref_linear(x, w, None, torch.bfloat16).float(), atol=2e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_silu_mul(ops, dtype):
+    torch.manual_seed(5)
+    inter = 176
+    x = torch.randn(33, 64, device=DEV).to(dtype)
+    w = (torch.randn(2 * inter, 64, device=DEV) / 8).to(dtype)
+    y = ops[dtype].linear_silu_mul(x, w, inter)
+    gu = ref.ref_linear(x, w, None, torch.float64)
+    expect = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    torch.testing.assert_close(y.double(), expect, **tol(dtype))
+    # gate first, then up: swapping the halves must change the result
+    swapped = torch.nn.functional.silu(gu[:, inter:]) * gu[:, :inter]
+    assert (y.double() - swapped).abs().max() > 10 * (y.double() - expect).abs().max()
+
+
+# ----------------------------------------------------------------- rotary + kv
+def make_cache(pages, Hkv, page, D, dtype):
+    k = torch.randn(pages, Hkv, page, D, device=DEV).to(dtype)
+    return k, torch.randn(pages, Hkv, page, D, device=DEV).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("geom", [(4, 2, 16, 16), (3, 1, 32, 32), (5, 5, 48, 24), (32, 4, 64, 64), (7, 7, 128, 0)])
+def test_rotary_kv_store(ops, dtype, geom):
+    from mini_inference_engine_amd.parts.rope import rotary_tables
+    Hq, Hkv, D, rot = geom
+    torch.manual_seed(D)
+    T, page, pages = 37, 16, 40
+    cos, sin = rotary_tables(10000.0, rot, 700) if rot else (None, None)
+    if rot:
+        cos, sin = cos.to(DEV), sin.to(DEV)
+    qkv = torch.randn(T, (Hq + 2 * Hkv) * D, device=DEV).to(dtype)
+    pos = torch.randint(0, 700, (T,), device=DEV, dtype=torch.int32)
+    slots = (torch.randperm((pages - 1) * page, device=DEV)[:T] + page).to(torch.int32)
+    kc, vc = make_cache(pages, Hkv, page, D, dtype)
+    q_ref, kc_ref, vc_ref = qkv.clone(), kc.clone(), vc.clone()
+    ref.ref_rotary_kv_store(q_ref, pos, cos, sin, rot, Hq, Hkv, D, kc_ref, vc_ref, slots)
+    ops[dtype].rotary_kv_store(qkv, pos, cos, sin, rot, Hq, Hkv, D, kc, vc, slots)
+    torch.testing.assert_close(qkv.float(), q_ref.float(), **tol(dtype))
+    torch.testing.assert_close(kc.float(), kc_ref.float(), **tol(dtype))
+    assert torch.equal(vc, vc_ref), "values are copied, not computed"
+    assert torch.equal(kc[0], kc_ref[0]) and torch.equal(vc[0], vc_ref[0])
+
+
+def test_rotary_q_only(ops):
+    from mini_inference_engine_amd.parts.rope import rotary_tables
+    cos, sin = (t.to(DEV) for t in rotary_tables(500000.0, 32, 100))
+    q = torch.randn(11, 3 * 32, device=DEV)
+    pos = torch.arange(11, device=DEV, dtype=torch.int32) * 9
+    expect = q.clone()
+    ref.ref_rotary_kv_store(expect, pos, cos, sin, 32, 3, 0, 32, None, None, None)
+    ops[torch.float32].rotary_kv_store(q, pos, cos, sin, 32, 3, 0, 32, None, None, None)
+    torch.testing.assert_close(q, expect, atol=1e-6, rtol=1e-5)
+
+
+# ------------------------------------------------------------------ attention
+def paged_setup(ctx_lens, q_lens, Hq, Hkv, D, page, dtype, num_pages=None, seed=0, spike=None):
+    """Rows with ctx_lens[i] keys of which the last q_lens[i] are this step's tokens.  Pages are a
+    random permutation (page 0 never used); unused block-table entries are 0.
+    spike = (row, key): that key's k is made to dominate the row's last query."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    rows = len(ctx_lens)
+    need = sum(-(-c // page) for c in ctx_lens)
+    num_pages = num_pages or need + 5
+    kc = torch.randn(num_pages, Hkv, page, D, generator=g).to(dtype)
+    vc = torch.randn(num_pages, Hkv, page, D, generator=g).to(dtype)
+    perm = torch.randperm(num_pages - 1, generator=g) + 1
+    max_blocks = max(-(-c // page) for c in ctx_lens) + 2
+    bt = torch.zeros(rows, max_blocks, dtype=torch.int32)
+    i = 0
+    for r, c in enumerate(ctx_lens):
+        n = -(-c // page)
+        bt[r, :n] = perm[i:i + n]
+        i += n
+    T = sum(q_lens)
+    q = torch.randn(T, Hq * D, generator=g).to(dtype)
+    token_row = torch.repeat_interleave(torch.arange(rows), torch.tensor(q_lens)).to(torch.int32)
+    positions = torch.cat([torch.arange(c - n, c) for c, n in zip(ctx_lens, q_lens)]).to(torch.int32)
+    if spike is not None:
+        r, key = spike
+        t_last = sum(q_lens[:r + 1]) - 1
+        pg, off = int(bt[r, key // page]), key % page
+        direction = torch.randn(D, generator=g)
+        direction = direction / direction.norm()
+        kc[pg, :, off, :] = (direction * 6.0).to(dtype)
+        q[t_last] = (direction * 6.0).repeat(Hq).to(dtype)
+    step = SimpleNamespace(token_row=token_row.to(DEV), positions=positions.to(DEV), num_rows=rows,
+                           max_context=max(ctx_lens), num_tokens=T, num_decode_rows=sum(1 for n in q_lens if n == 1),
+                           max_row_tokens=max(q_lens), row_start=None)
+    group = SimpleNamespace(block_tables=bt.to(DEV), max_blocks=max_blocks)
+    return q.to(DEV), kc.to(DEV), vc.to(DEV), group, step
+
+
+def run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, scale, window):
+    out = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, scale, window)
+    expect = ref.ref_paged_attention(q, Hq, Hkv, D, kc, vc, group.block_tables, step.token_row, step.positions,
+                                     scale, window, torch.float64)
+    return out, expect
+
+
+ATT_TOL = {torch.float32: dict(atol=3e-6, rtol=1e-5), torch.bfloat16: dict(atol=2e-2, rtol=2e-2)}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ctx", [[1], [17], [1000], [2048], [5, 300, 1, 2047, 64, 65], list(range(1, 200, 7))])
+def test_decode_attention_reference_vectors(ops, dtype, ctx):
+    Hq, Hkv, D, page = 32, 4, 64, 16
+    q, kc, vc, group, step = paged_setup(ctx, [1] * len(ctx), Hq, Hkv, D, page, dtype, num_pages=4096)
+    out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1 / math.sqrt(D), None)
+    torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("geom", [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 16), (6, 2, 80, 32), (8, 1, 128, 64),
+                                  (2, 2, 256, 16), (12, 4, 96, 16)])
+def test_attention_mixed_rows(ops, dtype, geom):
+    """Single tokens beside portions that start anywhere, other head sizes, groups and page sizes."""
+    Hq, Hkv, D, page = geom
+    ctx = [40, 1, 16, 17, 130, 64, 33, 2]
+    qn = [1, 1, 1, 1, 50, 64, 2, 2]
+    q, kc, vc, group, step = paged_setup(ctx, qn, Hq, Hkv, D, page, dtype, seed=D)
+    out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 0.7 / math.sqrt(D), None)
+    torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("key", [0, 15, 16, 31, 255, 256, 700, 1022])
+def test_attention_finds_a_far_key(ops, dtype, key):
+    """One key among a thousand dominates: the output must be (nearly) that key's value, so a
+    kernel that skips a page edge, the first key or a split's last key fails by a wide margin."""
+    Hq, Hkv, D, page = 8, 2, 64, 16
+    ctx = [1023, 300]
+    q, kc, vc, group, step = paged_setup(ctx, [1, 1], Hq, Hkv, D, page, dtype, seed=key, spike=(0, key))
+    out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1.0, None)
+    pg, off = int(group.block_tables[0, key // page]), key % page
+    v_key = vc[pg, :, off, :].double().repeat_interleave(Hq // Hkv, 0).reshape(-1)
+    assert (expect[0] - v_key).abs().max() < 1e-3, "the set-up must make that key dominate"
+    torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 100])
+def test_attention_window_edge(ops, dtype, window):
+    """The key just outside the window dominates if it is (wrongly) seen; the one just inside must be."""
+    Hq, Hkv, D, page = 4, 2, 32, 16
+    ctx, qn = [200, 90], [1, 30]
+    for inside in (True, False):
+        key = 199 - window + 1 if inside else 199 - window
+        if key < 0:
+            continue
+        q, kc, vc, group, step = paged_setup(ctx, qn, Hq, Hkv, D, page, dtype, seed=window, spike=(0, key))
+        out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1.0, window)
+        torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+
+
+def test_attention_one_key_is_its_value(ops):
+    q, kc, vc, group, step = paged_setup([1, 1, 1], [1, 1, 1], 6, 3, 48, 16, torch.float32, seed=9)
+    out = ops[torch.float32].paged_attention(q, 6, 3, 48, kc, vc, group, step, 0.3, None)
+    for r in range(3):
+        v = vc[int(group.block_tables[r, 0]), :, 0, :].repeat_interleave(2, 0).reshape(-1)
+        torch.testing.assert_close(out[r], v, atol=1e-6, rtol=1e-6)
+
+
+def test_attention_ignores_stale_pages(ops):
+    """NaN in every slot beyond a row's context, and in pages it does not own, changes nothing."""
+    Hq, Hkv, D, page = 4, 2, 32, 16
+    ctx, qn = [37, 5, 64], [1, 5, 20]
+    q, kc, vc, group, step = paged_setup(ctx, qn, Hq, Hkv, D, page, torch.float32, seed=2)
+    clean = ops[torch.float32].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 0.2, None)
+    owned = torch.zeros(kc.shape[0], page, dtype=torch.bool, device=DEV)
+    for r, c in enumerate(ctx):
+        for p in range(c):
+            owned[int(group.block_tables[r, p // page]), p % page] = True
+    kc2, vc2 = kc.clone(), vc.clone()
+    kc2.permute(0, 2, 1, 3)[~owned] = float("nan")
+    vc2.permute(0, 2, 1, 3)[~owned] = float("nan")
+    dirty = ops[torch.float32].paged_attention(q, Hq, Hkv, D, kc2, vc2, group, step, 0.2, None)
+    assert torch.equal(clean, dirty)
+
+
+# ------------------------------------------------------------------- sampling
+def test_sample_greedy_and_ties(ops):
+    torch.manual_seed(0)
+    logits = torch.randn(9, 331, device=DEV)
+    logits[3, 100] = logits[3, 200] = 50.0          # equal maxima: the lowest index wins
+    logits[4] = 0.0
+    zeros = torch.zeros(9, device=DEV)
+    out = ops[torch.float32].sample(logits, zeros, torch.zeros(9, dtype=torch.int64, device=DEV),
+                                    torch.zeros(9, dtype=torch.int32, device=DEV))
+    expect = logits.argmax(-1)
+    expect[3], expect[4] = 100, 0
+    assert out.tolist() == expect.tolist()
+
+
+def test_sample_noise_matches_specification(ops):
+    torch.manual_seed(1)
+    V = 1000
+    logits = torch.randn(6, V, device=DEV) * 2
+    temps = torch.tensor([0.8, 0.0, 1.5, 0.8, 0.3, 1.0], device=DEV)
+    seeds = torch.tensor([1, 2, 2**40 + 3, 1, -5, 2**62], dtype=torch.int64, device=DEV)
+    ctrs = torch.tensor([0, 5, 7, 1, 2**31 - 1, 3], dtype=torch.int32, device=DEV)
+    out = ops[torch.float32].sample(logits, temps, seeds, ctrs).tolist()
+    for r in range(6):
+        z = ref.ref_perturbed(logits[r], float(temps[r]), int(seeds[r]), int(ctrs[r]))
+        # the kernel's float32 noise may differ from the float64 one in the last digits
+        assert float(z.max() - z[out[r]]) <= 1e-4, f"row {r}: chose {out[r]}, best {int(z.argmax())}"
+    assert out[0] != out[3] or True     # different counters draw different noise (not necessarily tokens)
+
+
+def test_sample_distribution(ops):
+    """Frequencies of the draw follow softmax(logits / t): chi-square on a small vocabulary."""
+    V, n, t = 7, 4000, 0.7
+    logits_row = torch.tensor([0.1, 1.0, -0.5, 2.0, 0.0, 1.5, -2.0], device=DEV)
+    logits = logits_row.repeat(n, 1).contiguous()
+    out = ops[torch.float32].sample(logits, torch.full((n,), t, device=DEV),
+                                    torch.full((n,), 1234, dtype=torch.int64, device=DEV),
+                                    torch.arange(n, dtype=torch.int32, device=DEV))
+    counts = torch.bincount(out.long().cpu(), minlength=V).double()
+    p = torch.softmax(logits_row.double().cpu() / t, 0)
+    chi2 = float(((counts - n * p) ** 2 / (n * p)).sum())
+    assert chi2 < 22.46, f"chi-square {chi2:.1f} with 6 degrees of freedom (p < 0.001 above 22.46)"
