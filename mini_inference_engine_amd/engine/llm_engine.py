@@ -148,10 +148,6 @@ class LLMEngine:
         if len(params) != len(prompts):
             raise ValueError(f"{len(prompts)} prompts but {len(params)} sampling params")
         seqs = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
-        done_early = [s for s in seqs if s.params.max_tokens == 0]
-        for s in done_early:                     # nothing to generate: never scheduled
-            self.scheduler.waiting.remove(s)
-            s.finish_time = s.first_token_time = time.perf_counter()
         while self.scheduler.has_work():
             self.step()
         outs = []

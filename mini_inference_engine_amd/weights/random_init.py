@@ -17,10 +17,12 @@ from safetensors.torch import save_file
 from ..config.registry import architecture_of
 
 
-def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std: float = 0.02) -> dict:
+def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std: float = 0.02, device="cpu") -> dict:
+    """``device`` other than the CPU draws from that device's generator (other values,
+    same distribution): for large benchmark models only."""
     from ..models.decoder import Decoder
     model = Decoder(architecture_of(config).build(config))
-    gen = torch.Generator(device="cpu").manual_seed(int(seed))
+    gen = torch.Generator(device=device).manual_seed(int(seed))
     out = {}
     for _, spec in model.param_specs():
         for s in spec.sources:
@@ -28,7 +30,7 @@ def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std: 
                 continue
             if spec.integer:
                 raise NotImplementedError("random integer tables")
-            t = torch.randn(s.shape, generator=gen, dtype=torch.float32) * std
+            t = torch.randn(s.shape, generator=gen, dtype=torch.float32, device=device) * std
             if len(s.shape) == 1:
                 t = t + 1.0
             out[s.name] = t.to(dtype).contiguous()
