@@ -1,8 +1,10 @@
 """Device tensors behind the cache manager's ids.
 
-One K and one V tensor per cache-owning layer call, [pages, kv_heads, page, head_dim]:
-the keys of one kv head within a page are one contiguous run (page * head_dim
-elements), which is what the attention kernels stream.  (The reference keeps
+One K and one V tensor per cache-owning layer call.  Keys: [pages, kv_heads, page, head_dim],
+so the keys of one kv head within a page are one contiguous run.  Values:
+[pages, kv_heads, head_dim, page], a page's values transposed, so that for one dim the
+page's keys are contiguous: both are then what the attention kernels' matrix
+instructions take straight from memory.  (The reference keeps
 [L, 2, pages, page, kv_heads, head_dim], inference_engine/model.py:43.)  State
 entries are [slots, *shape].
 """
@@ -32,9 +34,10 @@ class CacheStorage:
         for e, ce in model.cache_entries.items():
             r = ce.requirement
             if isinstance(r, PagedKV):
-                shape = (pages_per_group[ce.group], r.num_kv_heads, page_size, r.head_dim)
-                self.entries[e] = EntryTensors(ce.group, torch.zeros(shape, dtype=dtype, device=device),
-                                               torch.zeros(shape, dtype=dtype, device=device), None, page_size)
+                k_shape = (pages_per_group[ce.group], r.num_kv_heads, page_size, r.head_dim)
+                v_shape = (pages_per_group[ce.group], r.num_kv_heads, r.head_dim, page_size)
+                self.entries[e] = EntryTensors(ce.group, torch.zeros(k_shape, dtype=dtype, device=device),
+                                               torch.zeros(v_shape, dtype=dtype, device=device), None, page_size)
             elif isinstance(r, FixedState):
                 sd = torch.float32 if r.dtype == "float32" else dtype
                 self.entries[e] = EntryTensors(None, None, None, torch.zeros((num_state_slots, *r.shape), dtype=sd,

@@ -3,7 +3,8 @@
 //
 // One wavefront per (token, query head).  The token sits in row r at absolute position p and
 // sees keys lo..p of its own request, lo = max(0, p - window + 1) or 0, found through the
-// row's block table in caches laid out [pages, Hkv, page, D].  Keys are taken 64 at a time
+// row's block table in caches laid out [pages, Hkv, page, D] (keys) and [pages, Hkv, D, page]
+// (values, transposed within a page).  Keys are taken 64 at a time
 // (one per lane: q . k in increasing d), the softmax is kept online in 32-bit, and the 64
 // probabilities then weight the value rows with the lanes spread over D.  The order of every
 // sum depends only on (lo, p): the result for a token is bit-identical whatever else the
@@ -42,7 +43,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
                        int Hkv, int D, int page, float scale, int window) {
   __shared__ float qs[ATT_MAX_D];
   __shared__ float ps[64];
-  __shared__ long long base[64];
+  __shared__ long long base[64];     // per key of the chunk: offset of its value column
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int row = token_row[t], pos = positions[t];
   const int kvh = h / (Hq / Hkv);
@@ -65,7 +66,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
     if (valid) {
       const int pg = bt[key / page];
       const long long off = (((long long)pg * Hkv + kvh) * page + key % page) * D;
-      base[lane] = off;
+      base[lane] = ((long long)pg * Hkv + kvh) * page * D + key % page;
       const typename P::V* kp = reinterpret_cast<const typename P::V*>(k_cache + off);
       float dot = 0.f;
       for (int d0 = 0; d0 < D; d0 += P::N) {
@@ -91,7 +92,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
 #pragma unroll
       for (int i = 0; i < ATT_MAX_D / 64; ++i) {
         const int d = lane + 64 * i;
-        if (d < D) acc[i] = fmaf(pj, to_float(vp[d]), acc[i]);
+        if (d < D) acc[i] = fmaf(pj, to_float(vp[(size_t)d * page]), acc[i]);
       }
     }
     __syncthreads();

@@ -1,0 +1,272 @@
+// bfloat16 attention on the matrix cores of gfx950, for one head size per build (-DHEAD_DIM=N, a
+// multiple of 16 up to 256).  Caches: keys [pages, Hkv, page, D], values [pages, Hkv, D, page].
+//
+// decode_attention: single-token rows.  One workgroup per (row, kv head, 16 query heads of its group,
+// split of the context); its waves take 32-key blocks of the split in turn.  With v_mfma_f32_16x16x32_bf16
+//   S^T[key, head]  = K[key, d]  . Q^T[d, head]      A = 16 keys x 32 dims, straight from the key page
+//   O^T[d, head]   += V^T[d, key] . P^T[key, head]   A = 16 dims x 32 keys, straight from the value page
+// The scores come out with lane % 16 = head and 4 consecutive keys per lane group; that is already
+// the layout P^T needs as the B operand of the second product if the 32 keys of its reduction are
+// taken in the order (lane group, tile, i), and the value operand is loaded in that same order, so the
+// probabilities never leave registers.  Softmax state (max, sum) is one value per lane (its head);
+// exponentials are base 2 with scale * log2(e) folded into the scores.  The waves of a workgroup are
+// merged through LDS; splits write normalised partials and base-2 log-sum-exps, merged by a second
+// kernel.  Keys outside [lo, p] get probability 0 by selection and their values are zeroed, so stale
+// or poisoned slots never reach the sums.
+#include "common.hpp"
+
+#ifndef HEAD_DIM
+#error "build with -DHEAD_DIM=<multiple of 16>"
+#endif
+#if HEAD_DIM % 16 != 0 || HEAD_DIM < 16 || HEAD_DIM > 256
+#error "HEAD_DIM must be a multiple of 16 from 16 to 256"
+#endif
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int D = HEAD_DIM;
+constexpr int KS = (D + 31) / 32;      // 32-dim steps of q . k
+constexpr int DT = D / 16;             // 16-dim tiles of the output
+constexpr int NW = D > 128 ? 2 : 4;    // waves per workgroup (bounded by the LDS the merge needs)
+constexpr int BLOCK_KEYS = 32;
+
+union Frag {
+  bf16x8 v;
+  uint4 q;
+  uint2 h[2];
+  uint32_t w[4];
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  // round to nearest even, low half = a
+  uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+  ua += 0x7FFFu + ((ua >> 16) & 1u);
+  ub += 0x7FFFu + ((ub >> 16) & 1u);
+  return (ua >> 16) | (ub & 0xFFFF0000u);
+}
+
+__global__ void __launch_bounds__(NW * 64)
+decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* __restrict__ k_cache,
+                        const bf16* __restrict__ v_cache, bf16* __restrict__ out, float* __restrict__ o_part,
+                        float* __restrict__ lse_part, const int* __restrict__ block_tables, int max_blocks,
+                        const int* __restrict__ positions, int Hq, int Hkv, int head_tiles, int page,
+                        float scale_log2, int window, int partition, int num_splits) {
+  __shared__ float s_m[NW][16], s_l[NW][16], s_M[16], s_L[16];
+  __shared__ float s_o[NW][16][D + 1];
+  const int b = blockIdx.x;
+  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
+  const int s = blockIdx.z;
+  const int G = Hq / Hkv;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, kb = lane >> 4;
+  const int pos = positions[b];
+  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  const int begin = (lo & ~(BLOCK_KEYS - 1)) + s * partition;
+  const int end = begin + partition < pos + 1 ? begin + partition : pos + 1;
+  const int g = ht * 16 + col;
+  const bool head_ok = g < G;
+  const int head = kvh * G + (head_ok ? g : 0);
+
+  if (begin > pos) {          // this split lies beyond the row's keys (uniform over the workgroup)
+    if (num_splits > 1 && threadIdx.x < 16 && ht * 16 + (int)threadIdx.x < G)
+      lse_part[((size_t)b * Hq + kvh * G + ht * 16 + threadIdx.x) * num_splits + s] = -INFINITY;
+    return;
+  }
+
+  const int* bt = block_tables + (size_t)b * max_blocks;
+  Frag qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d0 = ks * 32 + kb * 8;
+    qf[ks].q = make_uint4(0, 0, 0, 0);
+    if (head_ok && d0 < D) qf[ks].q = *reinterpret_cast<const uint4*>(q + (size_t)b * q_stride + (size_t)head * D + d0);
+  }
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 O[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) O[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int blk = begin + BLOCK_KEYS * wave; blk < end; blk += BLOCK_KEYS * NW) {
+    // ---- scores of 32 keys x 16 heads
+    f32x4 S[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      S[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      int key = blk + 16 * t + col;
+      key = key < pos ? key : pos;                      // never look up pages the row does not have
+      const int pg = bt[key / page];
+      const bf16* kp = k_cache + (((size_t)pg * Hkv + kvh) * page + key % page) * D;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = ks * 32 + kb * 8;
+        Frag a;
+        a.q = make_uint4(0, 0, 0, 0);
+        if (d0 < D) a.q = *reinterpret_cast<const uint4*>(kp + d0);
+        S[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[ks].v, S[t], 0, 0, 0);
+      }
+    }
+    // ---- values of the same 32 keys, in the order the probabilities sit in registers
+    const bool partial = blk + BLOCK_KEYS > pos + 1 || blk < lo;
+    Frag va[DT];
+    {
+      int k0 = blk + 4 * kb, k1 = blk + 16 + 4 * kb;
+      const int last = pos & ~3;
+      k0 = k0 < last ? k0 : last;
+      k1 = k1 < last ? k1 : last;
+      const int pg0 = bt[k0 / page], pg1 = bt[k1 / page];
+      const bf16* v0 = v_cache + ((size_t)pg0 * Hkv + kvh) * D * page + k0 % page;
+      const bf16* v1 = v_cache + ((size_t)pg1 * Hkv + kvh) * D * page + k1 % page;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const size_t drow = (size_t)(dt * 16 + col) * page;
+        va[dt].h[0] = *reinterpret_cast<const uint2*>(v0 + drow);
+        va[dt].h[1] = *reinterpret_cast<const uint2*>(v1 + drow);
+      }
+    }
+    // ---- online softmax, one head per lane column
+    float sv[8];
+    bool ok[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = blk + 16 * t + 4 * kb + i;
+        ok[t * 4 + i] = key >= lo && key <= pos;
+        sv[t * 4 + i] = ok[t * 4 + i] ? S[t][i] * scale_log2 : -INFINITY;
+        mx = fmaxf(mx, sv[t * 4 + i]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);                   // finite: every block taken holds a visible key
+    const float alpha = exp2f(m - m_new);
+    float p[8], rs = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      p[j] = ok[j] ? exp2f(sv[j] - m_new) : 0.f;
+      rs += p[j];
+    }
+    rs += __shfl_xor(rs, 16, 64);
+    rs += __shfl_xor(rs, 32, 64);
+    l = l * alpha + rs;
+    m = m_new;
+    Frag pb;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pb.w[j] = pack_bf16(p[2 * j], p[2 * j + 1]);
+    if (partial) {
+      // zero the values of keys outside [lo, pos]: 0 * (stale NaN) must not reach the sum
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t w = va[dt].w[j];
+          if (!ok[2 * j]) w &= 0xFFFF0000u;
+          if (!ok[2 * j + 1]) w &= 0x0000FFFFu;
+          va[dt].w[j] = w;
+        }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      O[dt] *= alpha;
+      O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt].v, pb.v, O[dt], 0, 0, 0);
+    }
+  }
+
+  // ---- merge the waves of the workgroup
+  if (kb == 0) {
+    s_m[wave][col] = m;
+    s_l[wave][col] = l;
+  }
+  __syncthreads();
+  float M = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) M = fmaxf(M, s_m[w][col]);
+  float L = 0.f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) {
+    const float mw = s_m[w][col];
+    L += mw == -INFINITY ? 0.f : exp2f(mw - M) * s_l[w][col];
+  }
+  const float f = m == -INFINITY ? 0.f : exp2f(m - M);
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s_o[wave][col][dt * 16 + 4 * kb + i] = O[dt][i] * f;
+  if (wave == 0 && kb == 0) {
+    s_M[col] = M;
+    s_L[col] = L;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 16 * D; e += NW * 64) {
+    const int hc = e / D, d = e - hc * D;
+    const int gg = ht * 16 + hc;
+    if (gg >= G) continue;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += s_o[w][hc][d];
+    const float val = sum / s_L[hc];
+    const size_t hh = (size_t)b * Hq + kvh * G + gg;
+    if (num_splits == 1) {
+      out[hh * D + d] = __float2bfloat16(val);
+    } else {
+      o_part[(hh * num_splits + s) * D + d] = val;
+      if (d == 0) lse_part[hh * num_splits + s] = s_M[hc] + log2f(s_L[hc]);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(64)
+merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ lse_part, bf16* __restrict__ out,
+                    int num_splits) {
+  const size_t hh = blockIdx.x;
+  const float* lse = lse_part + hh * num_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, lse[s]);
+  float W = 0.f;
+  for (int s = 0; s < num_splits; ++s) W += lse[s] == -INFINITY ? 0.f : exp2f(lse[s] - M);
+  const float inv = 1.0f / W;
+  for (int d = threadIdx.x; d < D; d += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < num_splits; ++s) {
+      const float ls = lse[s];
+      if (ls != -INFINITY) acc += exp2f(ls - M) * o_part[(hh * num_splits + s) * D + d];
+    }
+    out[hh * D + d] = __float2bfloat16(acc * inv);
+  }
+}
+
+MIE_EXPORT const char* attention_bf16_last_error() { return g_mie_error; }
+MIE_EXPORT int mie_attention_bf16_head_dim() { return D; }
+MIE_EXPORT int mie_decode_block_keys() { return BLOCK_KEYS * NW; }
+
+// q: token b is row b (single-token rows lead the flattened batch).  partition: keys per split, a
+// multiple of mie_decode_block_keys().  o_part [rows, Hq, splits, D] and lse_part [rows, Hq, splits]
+// float are needed when num_splits > 1.
+MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                    float* o_part, float* lse_part, const int* block_tables, int max_blocks,
+                                    const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
+                                    float scale, int window, int partition, int num_splits, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (head_dim != D) MIE_FAIL("decode_attention: built for head_dim %d, called with %d", D, head_dim);
+  if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("decode_attention: %d query heads on %d kv heads", Hq, Hkv);
+  if (page < 16 || page % 16) MIE_FAIL("decode_attention: page size %d (multiples of 16)", page);
+  if (partition <= 0 || partition % (BLOCK_KEYS * NW)) MIE_FAIL("decode_attention: partition %d is no multiple of %d", partition, BLOCK_KEYS * NW);
+  if (num_splits < 1 || num_splits > 65535) MIE_FAIL("decode_attention: %d splits", num_splits);
+  if (num_splits > 1 && (!o_part || !lse_part)) MIE_FAIL("decode_attention: splits need partial buffers");
+  if (q_stride < (long)Hq * D || (q_stride % 8) || ((uintptr_t)q % 16)) MIE_FAIL("decode_attention: q stride %ld / alignment", q_stride);
+  if (max_blocks <= 0) MIE_FAIL("decode_attention: max_blocks %d", max_blocks);
+  const int G = Hq / Hkv, head_tiles = (G + 15) / 16;
+  if ((long)Hkv * head_tiles > 65535) MIE_FAIL("decode_attention: too many head tiles for the grid");
+  dim3 grid(rows, Hkv * head_tiles, num_splits), block(NW * 64);
+  hipLaunchKernelGGL(decode_attention_kernel, grid, block, 0, stream, (const bf16*)q, q_stride, (const bf16*)k_cache,
+                     (const bf16*)v_cache, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv,
+                     head_tiles, page, scale * 1.4426950408889634f, window, partition, num_splits);
+  MIE_CHECK_LAUNCH("decode_attention");
+  if (num_splits > 1) {
+    hipLaunchKernelGGL(merge_splits_kernel, dim3(rows * Hq), dim3(64), 0, stream, o_part, lse_part, (bf16*)out, num_splits);
+    MIE_CHECK_LAUNCH("merge_splits");
+  }
+  return 0;
+}

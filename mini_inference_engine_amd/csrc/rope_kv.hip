@@ -6,7 +6,9 @@
 //   out[j]           = x[j] c - x[j + rot/2] s
 //   out[j + rot/2]   = x[j + rot/2] c + x[j] s            (computed in 32-bit, rounded once)
 // dims rot..D of a head are left as they are.  k (rotated) and v of token t go to slot
-// slot_mapping[t] of caches laid out [pages, Hkv, page, D].
+// slot_mapping[t]: keys into a cache laid out [pages, Hkv, page, D], values into one laid out
+// [pages, Hkv, D, page] (a page's values transposed: the 16+ keys of one dim are contiguous,
+// which is how the attention kernels' matrix instructions want them).
 #include "common.hpp"
 
 template <typename T>
@@ -18,10 +20,11 @@ rotary_kv_store_kernel(T* __restrict__ qkv, long row_stride, const int* __restri
   const int t = blockIdx.x;
   T* row = qkv + (size_t)t * row_stride;
   const int half = rot >> 1;
-  size_t k_base = 0;
+  size_t k_base = 0, v_base = 0;
   if (Hkv) {
     const int slot = slots[t];
     k_base = ((size_t)(slot / page) * Hkv * page + (size_t)(slot % page)) * D;   // + kvh * page * D
+    v_base = (size_t)(slot / page) * Hkv * page * D + (size_t)(slot % page);     // + (kvh * D + d) * page
   }
   if (half) {
     const int pos = positions[t];
@@ -52,7 +55,7 @@ rotary_kv_store_kernel(T* __restrict__ qkv, long row_stride, const int* __restri
     }
     for (int w = threadIdx.x; w < Hkv * D; w += blockDim.x) {
       const int kvh = w / D, d = w - kvh * D;
-      v_cache[k_base + (size_t)kvh * page * D + d] = row[(size_t)(Hq + Hkv + kvh) * D + d];
+      v_cache[v_base + ((size_t)kvh * D + d) * page] = row[(size_t)(Hq + Hkv + kvh) * D + d];
     }
   }
 }

@@ -37,7 +37,7 @@ class KernelBackend:
         """Rotate the first ``rotary_dim`` dims of every q and k head of
         qkv [T, (Hq + 2 Hkv) D] in place (pairs j, j + rotary_dim / 2; angle tables
         cos, sin [positions, rotary_dim / 2] float32), then write k and v of token t to
-        cache slot slot_mapping[t] of k_cache, v_cache [pages, Hkv, page, D].
+        cache slot slot_mapping[t] of k_cache [pages, Hkv, page, D] and v_cache [pages, Hkv, D, page].
         rotary_dim 0: no rotation.  num_kv_heads 0 (k_cache None): q only, no write."""
         raise NotImplementedError
 

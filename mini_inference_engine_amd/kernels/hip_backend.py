@@ -89,6 +89,13 @@ class HipBackend(KernelBackend):
             "sampling": {
                 "mie_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
             },
+            "attention_bf16": {
+                "mie_decode_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                         c_int, c_void_p],
+                "mie_decode_block_keys": [],
+                "mie_attention_bf16_head_dim": [],
+            },
         }.get(module, {})
         for name, argtypes in sig.items():
             fn = getattr(lib, name)
@@ -198,8 +205,8 @@ class HipBackend(KernelBackend):
                 raise ValueError("rotary_kv_store: positions must be contiguous int32 [T]")
         if Hkv:
             page = k_cache.shape[2]
-            want = (k_cache.shape[0], Hkv, page, D)
-            for name, t in (("k_cache", k_cache), ("v_cache", v_cache)):
+            for name, t, want in (("k_cache", k_cache, (k_cache.shape[0], Hkv, page, D)),
+                                  ("v_cache", v_cache, (k_cache.shape[0], Hkv, D, page))):
                 if tuple(t.shape) != want or t.dtype != qkv.dtype or not t.is_contiguous():
                     raise ValueError(f"rotary_kv_store: {name} {tuple(t.shape)} {t.dtype}, expected {want} {qkv.dtype}")
             if slot_mapping.dtype != torch.int32 or slot_mapping.shape[0] != T or not slot_mapping.is_contiguous():
@@ -215,7 +222,7 @@ class HipBackend(KernelBackend):
         if qkv.shape[1] < Hq * D:
             raise ValueError(f"paged_attention: qkv has {qkv.shape[1]} columns, fewer than {Hq * D}")
         pages, hk, page, d = k_cache.shape
-        if (hk, d) != (Hkv, D) or tuple(v_cache.shape) != tuple(k_cache.shape):
+        if (hk, d) != (Hkv, D) or tuple(v_cache.shape) != (pages, Hkv, D, page):
             raise ValueError(f"paged_attention: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for "
                              f"{Hkv} kv heads of {D}")
         if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype or not (k_cache.is_contiguous() and
@@ -234,17 +241,53 @@ class HipBackend(KernelBackend):
                              f"({bt.shape[1]} pages of {page})")
         return T, page, bt
 
+    # workgroups the decode attention kernel should at least be spread over (two per compute unit)
+    DECODE_TARGET_WORKGROUPS = 512
+
+    def decode_splits(self, rows: int, Hq: int, Hkv: int, context_bound: int, window, block_keys: int):
+        """(keys per split, number of splits) for single-token rows: split the context only as far
+        as the rows and heads alone do not fill the GPU (inference_engine/kernels/decode_attention.py:117-125
+        follows the same idea), in whole blocks of the kernel."""
+        if window:
+            context_bound = min(context_bound, window + 32)
+        base = rows * Hkv * -(-(Hq // Hkv) // 16)
+        most = max(1, -(-context_bound // block_keys))
+        splits = max(1, min(-(-self.DECODE_TARGET_WORKGROUPS // base), most))
+        partition = -(-(-(-context_bound // splits)) // block_keys) * block_keys
+        return partition, max(1, -(-context_bound // partition))
+
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
-                        window):
+                        window, force_generic: bool = False, num_splits: int | None = None):
         self._on_device(qkv, k_cache, v_cache)
         Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
         T, page, bt = self._check_attention(qkv, Hq, Hkv, D, k_cache, v_cache, group, step)
         out = torch.empty((T, Hq * D), dtype=qkv.dtype, device=qkv.device)
-        lib = self.lib("attention")
-        library.check(lib, lib.mie_paged_attention(
-            _ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _code(qkv.dtype), _ptr(bt),
-            bt.shape[1], _ptr(step.token_row), _ptr(step.positions), T, Hq, Hkv, D, page, float(scale),
-            int(window or 0), self._stream()))
+        done = 0
+        if qkv.dtype == torch.bfloat16 and not force_generic and step.num_decode_rows > 0:
+            done = step.num_decode_rows        # single-token rows lead the batch: token t is row t
+            lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))
+            block_keys = lib.mie_decode_block_keys()
+            partition, splits = self.decode_splits(done, Hq, Hkv, step.max_context, window, block_keys)
+            if num_splits is not None:
+                bound = min(step.max_context, window + 32) if window else step.max_context
+                partition = -(-(-(-bound // num_splits)) // block_keys) * block_keys
+                splits = max(1, -(-bound // partition))
+            o_part = lse_part = None
+            if splits > 1:
+                o_part = torch.empty((done, Hq, splits, D), dtype=torch.float32, device=qkv.device)
+                lse_part = torch.empty((done, Hq, splits), dtype=torch.float32, device=qkv.device)
+            library.check(lib, lib.mie_decode_attention(
+                _ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(o_part), _ptr(lse_part),
+                _ptr(bt), bt.shape[1], _ptr(step.positions), done, Hq, Hkv, D, page, float(scale), int(window or 0),
+                partition, splits, self._stream()))
+        if done < T:
+            lib = self.lib("attention")
+            esz = qkv.element_size()
+            library.check(lib, lib.mie_paged_attention(
+                c_void_p(qkv.data_ptr() + done * qkv.stride(0) * esz), qkv.stride(0), _ptr(k_cache), _ptr(v_cache),
+                c_void_p(out.data_ptr() + done * Hq * D * esz), _code(qkv.dtype), _ptr(bt), bt.shape[1],
+                c_void_p(step.token_row.data_ptr() + done * 4), c_void_p(step.positions.data_ptr() + done * 4),
+                T - done, Hq, Hkv, D, page, float(scale), int(window or 0), self._stream()))
         return out
 
     def sample(self, logits, temperatures, seeds, counters):

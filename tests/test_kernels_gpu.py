@@ -141,7 +141,7 @@ def test_linear_silu_mul(ops, dtype):
 # ----------------------------------------------------------------- rotary + kv
 def make_cache(pages, Hkv, page, D, dtype):
     k = torch.randn(pages, Hkv, page, D, device=DEV).to(dtype)
-    return k, torch.randn(pages, Hkv, page, D, device=DEV).to(dtype)
+    return k, torch.randn(pages, Hkv, D, page, device=DEV).to(dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -188,7 +188,7 @@ def paged_setup(ctx_lens, q_lens, Hq, Hkv, D, page, dtype, num_pages=None, seed=
     need = sum(-(-c // page) for c in ctx_lens)
     num_pages = num_pages or need + 5
     kc = torch.randn(num_pages, Hkv, page, D, generator=g).to(dtype)
-    vc = torch.randn(num_pages, Hkv, page, D, generator=g).to(dtype)
+    vc = torch.randn(num_pages, Hkv, D, page, generator=g).to(dtype)
     perm = torch.randperm(num_pages - 1, generator=g) + 1
     max_blocks = max(-(-c // page) for c in ctx_lens) + 2
     bt = torch.zeros(rows, max_blocks, dtype=torch.int32)
@@ -216,8 +216,8 @@ def paged_setup(ctx_lens, q_lens, Hq, Hkv, D, page, dtype, num_pages=None, seed=
     return q.to(DEV), kc.to(DEV), vc.to(DEV), group, step
 
 
-def run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, scale, window):
-    out = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, scale, window)
+def run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, scale, window, **kw):
+    out = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, scale, window, **kw)
     expect = ref.ref_paged_attention(q, Hq, Hkv, D, kc, vc, group.block_tables, step.token_row, step.positions,
                                      scale, window, torch.float64)
     return out, expect
@@ -237,6 +237,69 @@ def test_decode_attention_reference_vectors(ops, dtype, ctx):
     q, kc, vc, group, step = paged_setup(ctx, [1] * len(ctx), Hq, Hkv, D, page, dtype, num_pages=4096)
     out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1 / math.sqrt(D), None)
     torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+
+
+@pytest.mark.parametrize("splits", [None, 1, 3, 8])
+@pytest.mark.parametrize("ctx", [[1], [17], [1000], [2048], [5, 300, 1, 2047, 64, 65], list(range(1, 200, 7))])
+def test_decode_attention_split_count_and_static_bound(ops, ctx, splits):
+    """The matrix-core decode kernel: any split count, and a looser bound on the context (as under
+    graph capture, where the bound is static), give the same answer
+    (the reference tests the same: tests/test_kernels.py:54-59 there)."""
+    Hq, Hkv, D, page = 32, 4, 64, 16
+    dtype = torch.bfloat16
+    q, kc, vc, group, step = paged_setup(ctx, [1] * len(ctx), Hq, Hkv, D, page, dtype, num_pages=4096, seed=len(ctx))
+    out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1 / math.sqrt(D), None, num_splits=splits)
+    torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+    generic = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 1 / math.sqrt(D), None, force_generic=True)
+    torch.testing.assert_close(out.float(), generic.float(), **ATT_TOL[dtype])
+    step.max_context = 2048
+    group.block_tables = torch.nn.functional.pad(group.block_tables, (0, 2048 // page + 1 - group.block_tables.shape[1]))
+    out2 = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 1 / math.sqrt(D), None, num_splits=splits)
+    torch.testing.assert_close(out2.double(), expect, **ATT_TOL[dtype])
+
+
+@pytest.mark.parametrize("geom", [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 16), (40, 2, 80, 32), (8, 1, 128, 64),
+                                  (2, 2, 256, 16), (12, 4, 96, 48), (17, 1, 64, 16)])
+@pytest.mark.parametrize("window", [None, 40])
+def test_decode_attention_geometries(ops, geom, window):
+    """Other head sizes (steps of 16), groups beyond 16 heads, odd counts, page sizes, a window."""
+    Hq, Hkv, D, page = geom
+    ctx = [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 500, 96]
+    dtype = torch.bfloat16
+    q, kc, vc, group, step = paged_setup(ctx, [1] * len(ctx), Hq, Hkv, D, page, dtype, seed=D + Hq)
+    for splits in (None, 1, 4):
+        out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 0.9 / math.sqrt(D), window,
+                                    num_splits=splits)
+        torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+
+
+def test_decode_attention_ignores_stale_pages_bf16(ops):
+    Hq, Hkv, D, page = 8, 2, 64, 16
+    ctx = [37, 5, 64, 1, 130, 33]
+    dtype = torch.bfloat16
+    q, kc, vc, group, step = paged_setup(ctx, [1] * len(ctx), Hq, Hkv, D, page, dtype, seed=4)
+    owned = torch.zeros(kc.shape[0], page, dtype=torch.bool, device=DEV)
+    for r, c in enumerate(ctx):
+        for p in range(c):
+            owned[int(group.block_tables[r, p // page]), p % page] = True
+    kc2, vc2 = kc.clone(), vc.clone()
+    kc2.permute(0, 2, 1, 3)[~owned] = float("nan")
+    vc2.permute(0, 3, 1, 2)[~owned] = float("nan")
+    for splits in (1, 2):
+        clean = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 0.2, None, num_splits=splits)
+        dirty = ops[dtype].paged_attention(q, Hq, Hkv, D, kc2, vc2, group, step, 0.2, None, num_splits=splits)
+        assert torch.equal(clean, dirty)
+    for window in (3, 20):
+        clean = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 0.2, window)
+        lo_owned = owned.clone()
+        for r, c in enumerate(ctx):
+            for p in range(max(0, c - window)):
+                lo_owned[int(group.block_tables[r, p // page]), p % page] = False
+        kc3, vc3 = kc.clone(), vc.clone()
+        kc3.permute(0, 2, 1, 3)[~lo_owned] = float("nan")
+        vc3.permute(0, 3, 1, 2)[~lo_owned] = float("nan")
+        dirty = ops[dtype].paged_attention(q, Hq, Hkv, D, kc3, vc3, group, step, 0.2, window)
+        assert torch.equal(clean, dirty)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -262,7 +325,7 @@ def test_attention_finds_a_far_key(ops, dtype, key):
     q, kc, vc, group, step = paged_setup(ctx, [1, 1], Hq, Hkv, D, page, dtype, seed=key, spike=(0, key))
     out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1.0, None)
     pg, off = int(group.block_tables[0, key // page]), key % page
-    v_key = vc[pg, :, off, :].double().repeat_interleave(Hq // Hkv, 0).reshape(-1)
+    v_key = vc[pg, :, :, off].double().repeat_interleave(Hq // Hkv, 0).reshape(-1)
     assert (expect[0] - v_key).abs().max() < 1e-3, "the set-up must make that key dominate"
     torch.testing.assert_close(out.double(), expect, **SPIKE_TOL[dtype])
 
@@ -286,7 +349,7 @@ def test_attention_one_key_is_its_value(ops):
     q, kc, vc, group, step = paged_setup([1, 1, 1], [1, 1, 1], 6, 3, 48, 16, torch.float32, seed=9)
     out = ops[torch.float32].paged_attention(q, 6, 3, 48, kc, vc, group, step, 0.3, None)
     for r in range(3):
-        v = vc[int(group.block_tables[r, 0]), :, 0, :].repeat_interleave(2, 0).reshape(-1)
+        v = vc[int(group.block_tables[r, 0]), :, :, 0].repeat_interleave(2, 0).reshape(-1)
         torch.testing.assert_close(out[r], v, atol=1e-6, rtol=1e-6)
 
 
@@ -302,7 +365,7 @@ def test_attention_ignores_stale_pages(ops):
             owned[int(group.block_tables[r, p // page]), p % page] = True
     kc2, vc2 = kc.clone(), vc.clone()
     kc2.permute(0, 2, 1, 3)[~owned] = float("nan")
-    vc2.permute(0, 2, 1, 3)[~owned] = float("nan")
+    vc2.permute(0, 3, 1, 2)[~owned] = float("nan")
     dirty = ops[torch.float32].paged_attention(q, Hq, Hkv, D, kc2, vc2, group, step, 0.2, None)
     assert torch.equal(clean, dirty)
 

@@ -59,7 +59,7 @@ def ref_rotary_kv_store(qkv, positions, cos, sin, rotary_dim, Hq, Hkv, D, k_cach
         P = k_cache.shape[2]
         page, off = slot_mapping.long() // P, slot_mapping.long() % P
         k_cache[page, :, off, :] = heads[:, Hq:Hq + Hkv, :]
-        v_cache[page, :, off, :] = heads[:, Hq + Hkv:, :]
+        v_cache[page, :, :, off] = heads[:, Hq + Hkv:, :]       # values: [pages, Hkv, D, page]
 
 
 def ref_paged_attention(qkv, Hq, Hkv, D, k_cache, v_cache, block_tables, token_row, positions, scale, window,
@@ -78,7 +78,7 @@ def ref_paged_attention(qkv, Hq, Hkv, D, k_cache, v_cache, block_tables, token_r
         keys = torch.arange(lo, p + 1, device=qkv.device)
         pages = bt[rows[t], keys // P]
         k = k_cache[pages, :, keys % P, :].double()          # [n, Hkv, D]
-        v = v_cache[pages, :, keys % P, :].double()
+        v = v_cache[pages, :, :, keys % P].double()             # [n, Hkv, D]
         q = qkv[t, :Hq * D].double().view(Hkv, g, D)
         s = torch.einsum("hgd,nhd->hgn", q, k) * scale
         pr = torch.softmax(s, dim=-1)
