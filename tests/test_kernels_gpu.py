@@ -253,7 +253,8 @@ def test_decode_attention_split_count_and_static_bound(ops, ctx, splits):
     generic = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 1 / math.sqrt(D), None, force_generic=True)
     torch.testing.assert_close(out.float(), generic.float(), **ATT_TOL[dtype])
     step.max_context = 2048
-    group.block_tables = torch.nn.functional.pad(group.block_tables, (0, 2048 // page + 1 - group.block_tables.shape[1]))
+    extra = max(0, 2048 // page + 1 - group.block_tables.shape[1])
+    group.block_tables = torch.nn.functional.pad(group.block_tables, (0, extra)).contiguous()
     out2 = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 1 / math.sqrt(D), None, num_splits=splits)
     torch.testing.assert_close(out2.double(), expect, **ATT_TOL[dtype])
 
