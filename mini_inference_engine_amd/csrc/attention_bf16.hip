@@ -237,6 +237,186 @@ merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ 
   }
 }
 
+
+// prefill_attention: rows of several tokens, starting anywhere in their request.  The same two
+// products as above with "head" replaced by "query": S^T[key, query] = K . Q^T and
+// O^T[d, query] += V^T . P^T, so softmax state is again one value per lane (its query).  A wave owns
+// PF_NT tiles of 16 queries x 1 head (heads of one kv group and/or consecutive query tiles) and
+// walks the keys its queries can see in blocks of 32; each key and value fragment it loads feeds all
+// its tiles.  No LDS, no barriers: waves are independent.
+constexpr int PF_NT = D <= 64 ? 4 : (D <= 128 ? 2 : 1);
+
+__global__ void __launch_bounds__(256)
+prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* __restrict__ k_cache,
+                         const bf16* __restrict__ v_cache, bf16* __restrict__ out,
+                         const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ row_start,
+                         const int* __restrict__ row_position, int first_row, int Hq, int Hkv, int hpw,
+                         int head_chunks, int page, float scale_log2, int window) {
+  const int row = first_row + blockIdx.y;
+  const int kvh = blockIdx.z / head_chunks, hc = blockIdx.z - kvh * head_chunks;
+  const int G = Hq / Hkv;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, kb = lane >> 4;
+  const int t0 = row_start[row], q_len = row_start[row + 1] - t0, p0 = row_position[row];
+  const int qpw = PF_NT / hpw;                              // query tiles per wave
+  const int qt0 = (blockIdx.x * 4 + wave) * qpw;            // first query tile of this wave
+  if (qt0 * 16 >= q_len) return;
+  const int* bt = block_tables + (size_t)row * max_blocks;
+
+  bool tile_ok[PF_NT];
+  int qpos[PF_NT], qtok[PF_NT], tile_last[PF_NT], head[PF_NT];
+  bool q_ok[PF_NT];
+  Frag qf[PF_NT][KS];
+#pragma unroll
+  for (int j = 0; j < PF_NT; ++j) {
+    const int hq = j % hpw, qt = qt0 + j / hpw;
+    const int g = hc * hpw + hq;
+    tile_ok[j] = g < G && qt * 16 < q_len;
+    head[j] = kvh * G + (g < G ? g : 0);
+    int qi = qt * 16 + col;
+    q_ok[j] = tile_ok[j] && qi < q_len;
+    qi = qi < q_len ? qi : q_len - 1;
+    qtok[j] = t0 + qi;
+    qpos[j] = p0 + qi;
+    const int last_q = (qt * 16 + 15 < q_len ? qt * 16 + 15 : q_len - 1);
+    tile_last[j] = p0 + (last_q > 0 ? last_q : 0);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 32 + kb * 8;
+      qf[j][ks].q = make_uint4(0, 0, 0, 0);
+      if (tile_ok[j] && d0 < D)
+        qf[j][ks].q = *reinterpret_cast<const uint4*>(q + (size_t)qtok[j] * q_stride + (size_t)head[j] * D + d0);
+    }
+  }
+  int last_tok = (qt0 + qpw) * 16 - 1;
+  last_tok = last_tok < q_len ? last_tok : q_len - 1;
+  const int kmax = p0 + last_tok;                            // last key any query of this wave sees
+  int kmin = 0;
+  if (window > 0) {
+    kmin = p0 + qt0 * 16 - window + 1;
+    kmin = kmin > 0 ? kmin : 0;
+  }
+
+  float m[PF_NT], l[PF_NT];
+  f32x4 O[PF_NT][DT];
+#pragma unroll
+  for (int j = 0; j < PF_NT; ++j) {
+    m[j] = -INFINITY;
+    l[j] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) O[j][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int blk = kmin & ~(BLOCK_KEYS - 1); blk <= kmax; blk += BLOCK_KEYS) {
+    Frag a[2][KS];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      int key = blk + 16 * t + col;
+      key = key < kmax ? key : kmax;
+      const int pg = bt[key / page];
+      const bf16* kp = k_cache + (((size_t)pg * Hkv + kvh) * page + key % page) * D;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = ks * 32 + kb * 8;
+        a[t][ks].q = make_uint4(0, 0, 0, 0);
+        if (d0 < D) a[t][ks].q = *reinterpret_cast<const uint4*>(kp + d0);
+      }
+    }
+    Frag va[DT];
+    {
+      int k0 = blk + 4 * kb, k1 = blk + 16 + 4 * kb;
+      const int last = kmax & ~3;
+      k0 = k0 < last ? k0 : last;
+      k1 = k1 < last ? k1 : last;
+      const int pg0 = bt[k0 / page], pg1 = bt[k1 / page];
+      const bf16* v0 = v_cache + ((size_t)pg0 * Hkv + kvh) * D * page + k0 % page;
+      const bf16* v1 = v_cache + ((size_t)pg1 * Hkv + kvh) * D * page + k1 % page;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const size_t drow = (size_t)(dt * 16 + col) * page;
+        va[dt].h[0] = *reinterpret_cast<const uint2*>(v0 + drow);
+        va[dt].h[1] = *reinterpret_cast<const uint2*>(v1 + drow);
+      }
+      if (blk + BLOCK_KEYS > kmax + 1) {
+        // slots after the wave's last key may be stale: zero them (0 * NaN must not reach the sum)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) {
+            const int ka = blk + (jj < 2 ? 0 : 16) + 4 * kb + 2 * (jj & 1);
+            uint32_t w = va[dt].w[jj];
+            if (ka > kmax) w &= 0xFFFF0000u;
+            if (ka + 1 > kmax) w &= 0x0000FFFFu;
+            va[dt].w[jj] = w;
+          }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < PF_NT; ++j) {
+      if (!tile_ok[j] || blk > tile_last[j]) continue;       // uniform over the wave
+      f32x4 S[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        S[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          S[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][ks].v, qf[j][ks].v, S[t], 0, 0, 0);
+      }
+      const int hi = qpos[j];
+      const int lo = window > 0 ? hi - window + 1 : 0;
+      float sv[8];
+      bool ok[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = blk + 16 * t + 4 * kb + i;
+          ok[t * 4 + i] = key >= lo && key <= hi;
+          sv[t * 4 + i] = ok[t * 4 + i] ? S[t][i] * scale_log2 : -INFINITY;
+          mx = fmaxf(mx, sv[t * 4 + i]);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[j], mx);
+      // a query may see none of this block's keys (it lies before the block, or the block before its window)
+      const float alpha = m_new == -INFINITY ? 1.f : exp2f(m[j] - m_new);
+      float p[8], rs = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p[e] = ok[e] ? exp2f(sv[e] - m_new) : 0.f;
+        rs += p[e];
+      }
+      rs += __shfl_xor(rs, 16, 64);
+      rs += __shfl_xor(rs, 32, 64);
+      l[j] = l[j] * alpha + rs;
+      m[j] = m_new;
+      Frag pb;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pb.w[e] = pack_bf16(p[2 * e], p[2 * e + 1]);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        O[j][dt] *= alpha;
+        O[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt].v, pb.v, O[j][dt], 0, 0, 0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int j = 0; j < PF_NT; ++j) {
+    if (!q_ok[j]) continue;
+    const float inv = 1.0f / l[j];
+    bf16* op = out + ((size_t)qtok[j] * Hq + head[j]) * D + 4 * kb;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint2 st;
+      st.x = pack_bf16(O[j][dt][0] * inv, O[j][dt][1] * inv);
+      st.y = pack_bf16(O[j][dt][2] * inv, O[j][dt][3] * inv);
+      *reinterpret_cast<uint2*>(op + dt * 16) = st;
+    }
+  }
+}
+
 MIE_EXPORT const char* attention_bf16_last_error() { return g_mie_error; }
 MIE_EXPORT int mie_attention_bf16_head_dim() { return D; }
 MIE_EXPORT int mie_decode_block_keys() { return BLOCK_KEYS * NW; }
@@ -268,5 +448,34 @@ MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_
     hipLaunchKernelGGL(merge_splits_kernel, dim3(rows * Hq), dim3(64), 0, stream, o_part, lse_part, (bf16*)out, num_splits);
     MIE_CHECK_LAUNCH("merge_splits");
   }
+  return 0;
+}
+
+// Rows first_row .. first_row + rows - 1 of the step (those of more than one token).  q and out are
+// indexed by flat token; row_start [all rows + 1], row_position [all rows] as the step gives them.
+MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                     const int* block_tables, int max_blocks, const int* row_start,
+                                     const int* row_position, int first_row, int rows, int max_row_tokens, int Hq,
+                                     int Hkv, int head_dim, int page, float scale, int window, hipStream_t stream) {
+  if (rows <= 0 || max_row_tokens <= 0) return 0;
+  if (head_dim != D) MIE_FAIL("prefill_attention: built for head_dim %d, called with %d", D, head_dim);
+  if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("prefill_attention: %d query heads on %d kv heads", Hq, Hkv);
+  if (page < 16 || page % 16) MIE_FAIL("prefill_attention: page size %d (multiples of 16)", page);
+  if (q_stride < (long)Hq * D || (q_stride % 8) || ((uintptr_t)q % 16) || ((uintptr_t)out % 8))
+    MIE_FAIL("prefill_attention: q stride %ld / alignment", q_stride);
+  if (max_blocks <= 0) MIE_FAIL("prefill_attention: max_blocks %d", max_blocks);
+  const int G = Hq / Hkv;
+  int hpw = PF_NT;                       // heads of a kv group per wave: the largest power of two <= min(G, PF_NT)
+  while (hpw > G) hpw >>= 1;
+  if (G == 3 && PF_NT == 4) hpw = 4;     // three heads fit one wave with a tile to spare
+  const int head_chunks = (G + hpw - 1) / hpw;
+  const int queries_per_block = 4 * (PF_NT / hpw) * 16;
+  const long gx = (max_row_tokens + queries_per_block - 1) / queries_per_block;
+  if (rows > 65535 || (long)Hkv * head_chunks > 65535) MIE_FAIL("prefill_attention: grid too large (%d rows)", rows);
+  dim3 grid((unsigned)gx, rows, Hkv * head_chunks), block(256);
+  hipLaunchKernelGGL(prefill_attention_kernel, grid, block, 0, stream, (const bf16*)q, q_stride, (const bf16*)k_cache,
+                     (const bf16*)v_cache, (bf16*)out, block_tables, max_blocks, row_start, row_position, first_row,
+                     Hq, Hkv, hpw, head_chunks, page, scale * 1.4426950408889634f, window);
+  MIE_CHECK_LAUNCH("prefill_attention");
   return 0;
 }

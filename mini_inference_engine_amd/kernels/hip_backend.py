@@ -93,6 +93,9 @@ class HipBackend(KernelBackend):
                 "mie_decode_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                                          c_int, c_void_p],
+                "mie_prefill_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                          c_void_p],
                 "mie_decode_block_keys": [],
                 "mie_attention_bf16_head_dim": [],
             },
@@ -280,6 +283,19 @@ class HipBackend(KernelBackend):
                 _ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(o_part), _ptr(lse_part),
                 _ptr(bt), bt.shape[1], _ptr(step.positions), done, Hq, Hkv, D, page, float(scale), int(window or 0),
                 partition, splits, self._stream()))
+        if done < T and qkv.dtype == torch.bfloat16 and not force_generic:
+            # rows of several tokens: matrix-core kernel over their own and earlier portions' keys
+            for name, t, n in (("row_start", step.row_start, step.num_rows + 1),
+                               ("row_position", step.row_position, step.num_rows)):
+                if t is None or t.dtype != torch.int32 or t.shape[0] < n or not t.is_contiguous():
+                    raise ValueError(f"paged_attention: {name} must be contiguous int32 [{n}]")
+            lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))
+            library.check(lib, lib.mie_prefill_attention(
+                _ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(bt), bt.shape[1],
+                _ptr(step.row_start), _ptr(step.row_position), step.num_decode_rows,
+                step.num_rows - step.num_decode_rows, step.max_row_tokens, Hq, Hkv, D, page, float(scale),
+                int(window or 0), self._stream()))
+            done = T
         if done < T:
             lib = self.lib("attention")
             esz = qkv.element_size()

@@ -209,9 +209,16 @@ def paged_setup(ctx_lens, q_lens, Hq, Hkv, D, page, dtype, num_pages=None, seed=
         direction = direction / direction.norm()
         kc[pg, :, off, :] = (direction * 6.0).to(dtype)
         q[t_last] = (direction * 6.0).repeat(Hq).to(dtype)
+    nd = 0
+    while nd < rows and q_lens[nd] == 1:
+        nd += 1
+    assert all(n > 1 for n in q_lens[nd:]), "single-token rows lead the batch"
+    row_start = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    row_position = torch.tensor([c - n for c, n in zip(ctx_lens, q_lens)], dtype=torch.int32)
     step = SimpleNamespace(token_row=token_row.to(DEV), positions=positions.to(DEV), num_rows=rows,
-                           max_context=max(ctx_lens), num_tokens=T, num_decode_rows=sum(1 for n in q_lens if n == 1),
-                           max_row_tokens=max(q_lens), row_start=None)
+                           max_context=max(ctx_lens), num_tokens=T, num_decode_rows=nd,
+                           max_row_tokens=max(q_lens), row_start=row_start.to(DEV),
+                           row_position=row_position.to(DEV))
     group = SimpleNamespace(block_tables=bt.to(DEV), max_blocks=max_blocks)
     return q.to(DEV), kc.to(DEV), vc.to(DEV), group, step
 
@@ -344,6 +351,54 @@ def test_attention_window_edge(ops, dtype, window):
         q, kc, vc, group, step = paged_setup(ctx, qn, Hq, Hkv, D, page, dtype, seed=window, spike=(0, key))
         out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1.0, window)
         torch.testing.assert_close(out.double(), expect, **SPIKE_TOL[dtype])
+
+
+@pytest.mark.parametrize("geom", [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 16), (6, 2, 80, 32), (8, 1, 128, 64),
+                                  (2, 2, 256, 16), (12, 4, 96, 16), (32, 4, 64, 16), (8, 8, 128, 16)])
+@pytest.mark.parametrize("window", [None, 24])
+def test_prefill_attention_geometries(ops, geom, window):
+    """The matrix-core prefill kernel: portions that start anywhere (page edges, mid page), tails that
+    do not fill a tile, two-token rows, every head-size step, beside single-token rows."""
+    Hq, Hkv, D, page = geom
+    ctx = [9, 300, 2, 64, 65, 17, 200, 131, 48, 1000]
+    qn = [1, 1, 2, 64, 65, 17, 3, 100, 31, 489]
+    dtype = torch.bfloat16
+    q, kc, vc, group, step = paged_setup(ctx, qn, Hq, Hkv, D, page, dtype, seed=D * 3 + Hq)
+    out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1.1 / math.sqrt(D), window)
+    torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+    generic = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 1.1 / math.sqrt(D), window,
+                                         force_generic=True)
+    torch.testing.assert_close(out.float(), generic.float(), **ATT_TOL[dtype])
+
+
+def test_prefill_attention_ignores_stale_pages_bf16(ops):
+    Hq, Hkv, D, page = 8, 2, 64, 16
+    ctx, qn = [37, 5, 64, 130, 33], [30, 5, 2, 67, 33]
+    dtype = torch.bfloat16
+    q, kc, vc, group, step = paged_setup(ctx, qn, Hq, Hkv, D, page, dtype, seed=4)
+    owned = torch.zeros(kc.shape[0], page, dtype=torch.bool, device=DEV)
+    for r, c in enumerate(ctx):
+        for p in range(c):
+            owned[int(group.block_tables[r, p // page]), p % page] = True
+    kc2, vc2 = kc.clone(), vc.clone()
+    kc2.permute(0, 2, 1, 3)[~owned] = float("nan")
+    vc2.permute(0, 3, 1, 2)[~owned] = float("nan")
+    clean = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 0.2, None)
+    dirty = ops[dtype].paged_attention(q, Hq, Hkv, D, kc2, vc2, group, step, 0.2, None)
+    assert torch.equal(clean, dirty)
+
+
+def test_prefill_last_row_equals_decode(ops):
+    """The last token of a portion, computed by the prefill kernel, equals the same token computed as a
+    single-token row by the decode kernel (same keys, same cache), within bfloat16 rounding."""
+    Hq, Hkv, D, page = 8, 2, 64, 16
+    dtype = torch.bfloat16
+    q, kc, vc, group, step = paged_setup([150], [40], Hq, Hkv, D, page, dtype, seed=12)
+    whole = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, 0.125, None)
+    q1, _, _, g1, s1 = paged_setup([150], [1], Hq, Hkv, D, page, dtype, seed=12)
+    g1.block_tables = group.block_tables
+    last = ops[dtype].paged_attention(q[-1:].contiguous(), Hq, Hkv, D, kc, vc, g1, s1, 0.125, None)
+    torch.testing.assert_close(whole[-1:].float(), last.float(), **ATT_TOL[dtype])
 
 
 def test_attention_one_key_is_its_value(ops):
