@@ -9,6 +9,29 @@ Every op runs on the current stream and allocates its outputs with torch.
 from __future__ import annotations
 
 
+class Normed:
+    """A normalised input that is not computed yet: rmsnorm(residual (+ pending)) * weight, of all
+    rows or of ``rows``.  A backend's ``linear`` may take it whole (norm and product in one kernel);
+    anything else calls ``materialize()``, which also performs the pending add exactly once."""
+
+    def __init__(self, ops, pending, residual, weight, eps, rows=None):
+        self.ops, self.pending, self.residual, self.weight, self.eps, self.rows = ops, pending, residual, weight, eps, rows
+        self._value = None
+
+    @property
+    def shape(self):
+        n = self.residual.shape[0] if self.rows is None else self.rows.shape[0]
+        return (n, self.residual.shape[1])
+
+    def materialize(self, out_dtype=None):
+        if self._value is None:
+            self._value = self.ops.add_rmsnorm(self.pending, self.residual, self.weight, self.eps,
+                                               out_dtype=out_dtype, rows=self.rows)
+            if self.rows is None:
+                self.pending = None          # it is in the stream now
+        return self._value
+
+
 class KernelBackend:
     name = "?"
     act_dtype = None
@@ -24,12 +47,15 @@ class KernelBackend:
         computed, y is [len(rows), width] and residual is not modified."""
         raise NotImplementedError
 
-    def linear(self, x, w, bias=None, out_dtype=None):
-        """y = x w^T (+ bias); w [out, in]; 32-bit accumulation."""
+    def linear(self, x, w, bias=None, out_dtype=None, add_to=None):
+        """y = x w^T (+ bias); w [out, in]; 32-bit accumulation.  ``x`` is a tensor or a Normed.
+        With ``add_to`` (the float32 stream [T, out]) the backend may add y into it in place and
+        return None; if it returns a tensor, the caller still has to add it."""
         raise NotImplementedError
 
     def linear_silu_mul(self, x, w_gate_up, intermediate):
-        """gu = x w^T with w [2 * intermediate, in]; returns silu(gu[:, :I]) * gu[:, I:]."""
+        """gu = x w^T with w [2 * intermediate, in]; returns silu(gu[:, :I]) * gu[:, I:].
+        ``x`` is a tensor or a Normed."""
         raise NotImplementedError
 
     def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,

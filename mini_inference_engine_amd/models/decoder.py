@@ -109,5 +109,4 @@ class Decoder:
             h, residual = spec.layers[call.layer].forward(h, residual, step, binding)
         if step.num_logits == 0:
             return None
-        y = spec.final_norm.forward(h, residual, rows=step.logit_rows)
-        return spec.head.forward(y)
+        return spec.head.forward(spec.final_norm.lazy(h, residual, rows=step.logit_rows))

@@ -15,6 +15,8 @@ from .base import Mixer, PagedKV, ParamSpec, register_mixer
 
 @register_mixer("attention")
 class Attention(Mixer):
+    lazy_input = True
+
     def __init__(self, width: int, num_heads: int, num_kv_heads: int, head_dim: int, scale: float,
                  position, prefix: str, window: int | None = None, has_kv: bool = True):
         if num_heads % num_kv_heads:
@@ -50,7 +52,7 @@ class Attention(Mixer):
     def cache_requirement(self):
         return PagedKV(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x, step, cache):
+    def forward(self, x, step, cache, add_to=None):
         ops = self.ops
         if cache.read_only == self.has_kv:
             raise ValueError("an attention part with k/v projections owns its cache; one without reads another's")
@@ -61,4 +63,4 @@ class Attention(Mixer):
         self.position.encode_and_store(ops, qkv, step, self.num_heads, kv_heads_in_row, k_cache, v_cache, slots)
         out = ops.paged_attention(qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v,
                                   group, step, self.scale, self.window)
-        return ops.linear(out, self.w_o)
+        return ops.linear(out, self.w_o, add_to=add_to)

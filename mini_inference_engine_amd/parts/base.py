@@ -12,14 +12,18 @@ Norm.forward(x, residual, rows=None) -> y
     ``residual`` is the fp32 stream [T, width]; ``x`` (or None) is the branch
     output still to be added to it.  Adds in place, normalises, returns ``y`` in
     the activation dtype.  With ``rows`` (int32 indices) only those rows are
-    produced and the stream is left untouched.
+    produced and the stream is left untouched.  Norm.lazy(...) returns the same
+    as a kernels.api.Normed, for parts that set ``lazy_input`` and hand it to
+    their first ``ops.linear`` (norm and product then run as one kernel).
 PositionEncoding.encode_and_store(ops, qkv, step, layout, cache, slots)
     Encodes q and k inside the fused projection output in place, as a function of
     each token's absolute position only, and writes k, v to the cache.
-Mixer.forward(x, step, cache) -> y      [T, width] -> [T, width]
+Mixer.forward(x, step, cache, add_to=None) -> y or None     [T, width] -> [T, width]
     Must accept a portion that starts anywhere in a request and leave its cache
-    or state as if the request had been fed whole.
-FeedForward.forward(x, step) -> y       token-wise
+    or state as if the request had been fed whole.  ``add_to`` is the stream the
+    block will add y to: a part may pass it to its last ``ops.linear`` and return
+    what that returns (None = already added), or ignore it and return y.
+FeedForward.forward(x, step, add_to=None) -> y or None       token-wise
 Block.forward(h, residual, step, cache) -> (h, residual)
 """
 from __future__ import annotations
@@ -124,21 +128,29 @@ class Norm(Part):
     def forward(self, x, residual, rows=None):
         raise NotImplementedError
 
+    def lazy(self, x, residual, rows=None):
+        """The same result, deferred (kernels.api.Normed)."""
+        raise NotImplementedError
+
 
 class PositionEncoding(Part):
     pass
 
 
 class Mixer(Part):
+    lazy_input = False      # True: forward takes a Normed and gives it to its first ops.linear
+
     def cache_requirement(self):
         return None
 
-    def forward(self, x, step, cache: CacheBinding):
+    def forward(self, x, step, cache: CacheBinding, add_to=None):
         raise NotImplementedError
 
 
 class FeedForward(Part):
-    def forward(self, x, step):
+    lazy_input = False
+
+    def forward(self, x, step, add_to=None):
         raise NotImplementedError
 
 

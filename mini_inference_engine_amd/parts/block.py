@@ -22,7 +22,11 @@ class PreNormBlock(Block):
         return [self.norm_mixer, self.mixer, self.norm_feed_forward, self.feed_forward]
 
     def forward(self, h, residual, step, cache):
-        y = self.norm_mixer.forward(h, residual)
-        a = self.mixer.forward(y, step, cache)
-        y = self.norm_feed_forward.forward(a, residual)
-        return self.feed_forward.forward(y, step), residual
+        y = self.norm_mixer.lazy(h, residual)
+        if not self.mixer.lazy_input:
+            y = y.materialize()
+        a = self.mixer.forward(y, step, cache, add_to=residual)
+        y = self.norm_feed_forward.lazy(a, residual)
+        if not self.feed_forward.lazy_input:
+            y = y.materialize()
+        return self.feed_forward.forward(y, step, add_to=residual), residual

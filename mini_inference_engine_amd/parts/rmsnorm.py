@@ -7,6 +7,7 @@ The stream and every intermediate are 32-bit; y is rounded once.
 """
 from __future__ import annotations
 
+from ..kernels.api import Normed
 from .base import Norm, ParamSpec, register_norm
 
 
@@ -23,3 +24,6 @@ class RMSNorm(Norm):
 
     def forward(self, x, residual, rows=None, out_dtype=None):
         return self.ops.add_rmsnorm(x, residual, self.weight, self.eps, out_dtype=out_dtype, rows=rows)
+
+    def lazy(self, x, residual, rows=None):
+        return Normed(self.ops, x, residual, self.weight, self.eps, rows)

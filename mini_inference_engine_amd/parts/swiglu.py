@@ -8,6 +8,8 @@ from .base import FeedForward, ParamSpec, register_feed_forward
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
+    lazy_input = True
+
     def __init__(self, width: int, intermediate: int, prefix: str):
         self.width = int(width)
         self.intermediate = int(intermediate)
@@ -20,6 +22,6 @@ class SwiGLU(FeedForward):
         return [ParamSpec.stacked("w_gate_up", [(f"{p}.gate_proj.weight", (i, w)), (f"{p}.up_proj.weight", (i, w))]),
                 ParamSpec.single("w_down", f"{p}.down_proj.weight", (w, i))]
 
-    def forward(self, x, step):
+    def forward(self, x, step, add_to=None):
         a = self.ops.linear_silu_mul(x, self.w_gate_up, self.intermediate)
-        return self.ops.linear(a, self.w_down)
+        return self.ops.linear(a, self.w_down, add_to=add_to)

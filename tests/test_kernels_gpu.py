@@ -138,6 +138,95 @@ def test_linear_silu_mul(ops, dtype):
     assert (y.double() - swapped).abs().max() > 10 * (y.double() - expect).abs().max()
 
 
+# --------------------------------------------------- few-row fused products (bfloat16)
+def normed(ops, stream, w_norm, eps, rows=None, pending=None):
+    from mini_inference_engine_amd.kernels.api import Normed
+    return Normed(ops, pending, stream, w_norm, eps, rows)
+
+
+SKINNY_SHAPES = [(1, 64, 176), (7, 200, 331), (16, 2048, 2560), (17, 120, 96), (33, 5632, 2048), (64, 2048, 640),
+                 (8, 176, 64), (3, 96, 384)]
+
+
+@pytest.mark.parametrize("shape", SKINNY_SHAPES)
+def test_skinny_linear(ops, shape):
+    M, K, N = shape
+    o = ops[torch.bfloat16]
+    torch.manual_seed(M * 3 + N)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    assert o._skinny_ok(x, w, None), "this shape must take the fused kernel"
+    y = o.linear(x, w)
+    torch.testing.assert_close(y.float(), ref.ref_linear(x, w, None, torch.bfloat16).float(), atol=2e-2, rtol=1e-2)
+    y32 = o.linear(x, w, out_dtype=torch.float32)
+    torch.testing.assert_close(y32, ref.ref_linear(x, w, None, torch.float32), atol=2e-3, rtol=2e-3)
+    # a row's result does not depend on the rows beside it
+    for a, b in ((0, 1), (M // 2, M), (M - 1, M)):
+        assert torch.equal(o.linear(x[a:b].contiguous(), w, out_dtype=torch.float32), y32[a:b])
+    # residual add in the epilogue
+    stream = torch.randn(M, N, device=DEV)
+    expect = stream + ref.ref_linear(x, w, None, torch.float32)
+    assert o.linear(x, w, add_to=stream) is None
+    torch.testing.assert_close(stream, expect, atol=2e-3, rtol=2e-3)
+
+
+@pytest.mark.parametrize("w_norm_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", SKINNY_SHAPES)
+def test_skinny_norm_prologue(ops, shape, w_norm_dtype):
+    M, K, N = shape
+    o = ops[torch.bfloat16]
+    torch.manual_seed(M + N)
+    stream = torch.randn(M, K, device=DEV) * 3
+    g = (1 + 0.1 * torch.randn(K, device=DEV)).to(w_norm_dtype)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    before = stream.clone()
+    y = o.linear(normed(o, stream, g, 1e-5), w, out_dtype=torch.float32)
+    assert torch.equal(stream, before)
+    xn = ref.ref_add_rmsnorm(None, before.clone(), g, 1e-5, torch.float64)
+    expect = xn @ w.double().T
+    # x is rounded to bfloat16 once (8 bits), the products are summed in float32
+    torch.testing.assert_close(y.double(), expect, atol=2e-2, rtol=1e-2)
+    unfused = o.linear(o.add_rmsnorm(None, before.clone(), g, 1e-5), w, out_dtype=torch.float32)
+    torch.testing.assert_close(y, unfused, atol=2e-2, rtol=1e-2)
+
+
+def test_skinny_norm_prologue_gathers_rows(ops):
+    o = ops[torch.bfloat16]
+    torch.manual_seed(0)
+    stream = torch.randn(40, 96, device=DEV)
+    g = torch.randn(96, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(331, 96, device=DEV) / 10).to(torch.bfloat16)
+    rows = torch.tensor([39, 0, 7, 7, 21], device=DEV, dtype=torch.int32)
+    y = o.linear(normed(o, stream, g, 1e-6, rows=rows), w, out_dtype=torch.float32)
+    expect = ref.ref_add_rmsnorm(None, stream.clone(), g, 1e-6, torch.float64, rows) @ w.double().T
+    torch.testing.assert_close(y.double(), expect, atol=2e-2, rtol=1e-2)
+    # with something still to add, the fused kernel is not taken and the add happens exactly once
+    pending = torch.randn(40, 96, device=DEV).to(torch.bfloat16)
+    lazy = normed(o, stream.clone(), g, 1e-6, pending=pending)
+    y2 = o.linear(lazy, w[:, :], out_dtype=torch.float32)
+    y3 = o.linear(lazy, w[:, :], out_dtype=torch.float32)
+    assert torch.equal(y2, y3) and lazy.pending is None
+    torch.testing.assert_close(lazy.residual, stream + pending.float())
+
+
+@pytest.mark.parametrize("M, K, inter", [(1, 64, 176), (8, 2048, 5632), (20, 96, 256), (50, 120, 200), (64, 64, 48)])
+def test_skinny_swiglu(ops, M, K, inter):
+    o = ops[torch.bfloat16]
+    torch.manual_seed(inter)
+    stream = torch.randn(M, K, device=DEV)
+    g = (1 + 0.1 * torch.randn(K, device=DEV)).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, K, device=DEV) / math.sqrt(K) * 2).to(torch.bfloat16)
+    y = o.linear_silu_mul(normed(o, stream, g, 1e-5), w, inter)
+    xn = ref.ref_add_rmsnorm(None, stream.clone(), g, 1e-5, torch.float64)
+    gu = xn @ w.double().T
+    expect = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    torch.testing.assert_close(y.double(), expect, atol=3e-2, rtol=2e-2)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    y = o.linear_silu_mul(x, w, inter)
+    gu = x.double() @ w.double().T
+    torch.testing.assert_close(y.double(), torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:], atol=3e-2, rtol=2e-2)
+
+
 # ----------------------------------------------------------------- rotary + kv
 def make_cache(pages, Hkv, page, D, dtype):
     k = torch.randn(pages, Hkv, page, D, device=DEV).to(dtype)

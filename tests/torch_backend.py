@@ -12,7 +12,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from mini_inference_engine_amd.kernels.api import KernelBackend
+from mini_inference_engine_amd.kernels.api import KernelBackend, Normed
 
 
 def ref_embedding(ids, table):
@@ -123,8 +123,9 @@ def ref_sample(logits, temperatures, seeds, counters):
 class TorchBackend(KernelBackend):
     name = "torch-reference"
 
-    def __init__(self, act_dtype=torch.float32):
+    def __init__(self, act_dtype=torch.float32, adds_in_place=True):
         self.act_dtype = act_dtype
+        self.adds_in_place = adds_in_place      # linear(add_to=...) adds and returns None, or leaves it to the caller
         self.calls = {}
 
     def _count(self, name):
@@ -138,12 +139,20 @@ class TorchBackend(KernelBackend):
         self._count("add_rmsnorm")
         return ref_add_rmsnorm(x, residual, weight, eps, out_dtype or self.act_dtype, rows)
 
-    def linear(self, x, w, bias=None, out_dtype=None):
+    def linear(self, x, w, bias=None, out_dtype=None, add_to=None):
         self._count("linear")
-        return ref_linear(x, w, bias, out_dtype or self.act_dtype)
+        if isinstance(x, Normed):
+            x = x.materialize()
+        y = ref_linear(x, w, bias, out_dtype or self.act_dtype)
+        if add_to is not None and self.adds_in_place:
+            add_to.add_(y.float())
+            return None
+        return y
 
     def linear_silu_mul(self, x, w_gate_up, intermediate):
         self._count("linear_silu_mul")
+        if isinstance(x, Normed):
+            x = x.materialize()
         return ref_silu_mul(ref_linear(x, w_gate_up, None, self.act_dtype), intermediate, self.act_dtype)
 
     def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
