@@ -217,10 +217,15 @@ def test_skinny_swiglu(ops, M, K, inter):
     g = (1 + 0.1 * torch.randn(K, device=DEV)).to(torch.bfloat16)
     w = (torch.randn(2 * inter, K, device=DEV) / math.sqrt(K) * 2).to(torch.bfloat16)
     y = o.linear_silu_mul(normed(o, stream, g, 1e-5), w, inter)
-    xn = ref.ref_add_rmsnorm(None, stream.clone(), g, 1e-5, torch.float64)
-    gu = xn @ w.double().T
+    # The kernel's stated rounding: x = bfloat16(r * g), products summed in float32, the row's rstd applied to
+    # the sums, silu(gate) * up rounded once.  Mirroring that leaves summation order and the last rounding
+    # (2^-8 relative) as the only differences; silu(gate) * up amplifies input rounding by |up|, so a bound
+    # against the unrounded formula would have to scale with it (test_skinny_norm_prologue checks that side).
+    xb = (stream * g.float()).to(torch.bfloat16).double()
+    rstd = torch.rsqrt(stream.double().pow(2).mean(-1, keepdim=True) + 1e-5)
+    gu = (xb @ w.double().T) * rstd
     expect = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
-    torch.testing.assert_close(y.double(), expect, atol=3e-2, rtol=2e-2)
+    torch.testing.assert_close(y.double(), expect, atol=1e-3, rtol=1e-2)
     x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
     y = o.linear_silu_mul(x, w, inter)
     gu = x.double() @ w.double().T
