@@ -1,0 +1,223 @@
+"""Parts beyond Llama's, defined here and nowhere in the package: the engine must build and step
+them unchanged.  A toy architecture is registered from this file with
+
+  layer 0  a mixer with per-request state of fixed size (a decaying sum, no keys at all),
+  layer 1  attention with a window of 8 keys (its own page group; pages are released as the window passes),
+  layer 2  attention over all keys,
+  run order [0, 1, 2, 1, 3]: layer 1 runs twice (same weights, a cache of its own each time),
+  layer 3  attention without k/v projections that reads the cache of the run-order entry of layer 2,
+
+and a feed-forward of another kind in layer 0 (a gated product with tanh, no SiLU).  It is replayed in
+the four trace families against a plain whole-sequence implementation written out below.  The toy
+parts compute with torch on whatever device they are given; they are test fixtures, not models.
+"""
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+import plain_llama as plain
+import trace_util
+from torch_backend import TorchBackend
+
+from mini_inference_engine_amd.config import ModelConfig, register_architecture, unregister_architecture
+from mini_inference_engine_amd.engine.runner import ModelRunner
+from mini_inference_engine_amd.parts import (Attention, DecoderSpec, Embedding, FeedForward, FixedState, LayerCall,
+                                             LMHead, Mixer, ParamSpec, PreNormBlock, RMSNorm, RotaryHalfSplit, SwiGLU,
+                                             register_feed_forward, register_mixer)
+from mini_inference_engine_amd.replay.trace import replay
+from mini_inference_engine_amd.weights import random_tensors
+
+WIDTH, HEADS, KV, HD, INTER, VOCAB, WINDOW, DECAY = 48, 3, 1, 16, 80, 97, 8, 0.8
+
+
+@register_mixer("toy_decay")
+class DecayMixer(Mixer):
+    """s_t = decay * s_{t-1} + x_t per request, y_t = s_t W^T.  The state lives in the request's slot."""
+
+    def __init__(self, width, decay, prefix):
+        self.width, self.decay, self.prefix = width, decay, prefix
+        self.weight = None
+
+    def params(self):
+        return [ParamSpec.single("weight", f"{self.prefix}.weight", (self.width, self.width))]
+
+    def cache_requirement(self):
+        return FixedState((self.width,), "float32")
+
+    def forward(self, x, step, cache, add_to=None):
+        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        starts, first_pos, slots = step.host["row_start"], step.host["row_position"], step.host["state_slots"]
+        for r in range(step.num_rows):
+            a, b = int(starts[r]), int(starts[r + 1])
+            slot = int(slots[r])
+            s = cache.state[slot].clone() if first_pos[r] > 0 else torch.zeros_like(cache.state[slot])
+            for t in range(a, b):
+                s = self.decay * s + x[t].float()
+                out[t] = s
+            cache.state[slot] = s
+        return self.ops.linear(out.to(x.dtype), self.weight)
+
+
+@register_feed_forward("toy_tanh_gate")
+class TanhGate(FeedForward):
+    def __init__(self, width, inner, prefix):
+        self.width, self.inner, self.prefix = width, inner, prefix
+        self.w_in = self.w_out = None
+
+    def params(self):
+        return [ParamSpec.stacked("w_in", [(f"{self.prefix}.a.weight", (self.inner, self.width)),
+                                           (f"{self.prefix}.b.weight", (self.inner, self.width))]),
+                ParamSpec.single("w_out", f"{self.prefix}.out.weight", (self.width, self.inner))]
+
+    def forward(self, x, step, add_to=None):
+        ab = self.ops.linear(x, self.w_in).float()
+        h = torch.tanh(ab[:, :self.inner]) * ab[:, self.inner:]
+        return self.ops.linear(h.to(x.dtype), self.w_out, add_to=add_to)
+
+
+@dataclass(frozen=True)
+class ToyConfig(ModelConfig):
+    width: int = WIDTH
+    vocab: int = VOCAB
+    architecture = "ToyForCausalLM"
+
+    def to_dict(self):
+        return {"architectures": [self.architecture], "toy_width": self.width, "toy_vocab": self.vocab}
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(width=d["toy_width"], vocab=d["toy_vocab"])
+
+
+def build_toy(cfg: ToyConfig) -> DecoderSpec:
+    w = cfg.width
+    rope = RotaryHalfSplit(HD, 100.0, 256)
+
+    def norm(name):
+        return RMSNorm(w, 1e-5, name)
+
+    def attention(i, **kw):
+        return Attention(w, HEADS, KV, HD, scale=HD ** -0.5, position=rope, prefix=f"l{i}.att", **kw)
+
+    layers = [
+        PreNormBlock(norm("l0.n1"), DecayMixer(w, DECAY, "l0.mix"), norm("l0.n2"), TanhGate(w, 40, "l0.ff")),
+        PreNormBlock(norm("l1.n1"), attention(1, window=WINDOW), norm("l1.n2"), SwiGLU(w, INTER, "l1.ff")),
+        PreNormBlock(norm("l2.n1"), attention(2), norm("l2.n2"), SwiGLU(w, INTER, "l2.ff")),
+        PreNormBlock(norm("l3.n1"), attention(3, has_kv=False), norm("l3.n2"), SwiGLU(w, INTER, "l3.ff")),
+    ]
+    emb = Embedding(cfg.vocab, w, "emb")
+    return DecoderSpec(embedding=emb, layers=layers, final_norm=norm("out_norm"), head=LMHead(cfg.vocab, w, "head", emb),
+                       schedule=[LayerCall(0), LayerCall(1), LayerCall(2), LayerCall(1), LayerCall(3, cache_of=2)],
+                       max_position=256, vocab_size=cfg.vocab, eos_token_id=None)
+
+
+@pytest.fixture(scope="module")
+def toy():
+    register_architecture("ToyForCausalLM", ToyConfig, build_toy, replace=True)
+    cfg = ToyConfig()
+    # std 0.3 at width 48 gives scores with a standard deviation of about 4: far from uniform, so which
+    # keys are seen matters, yet not so sharp that float32 rounding of a score shows in the probabilities
+    weights = random_tensors(cfg, 9, torch.float32, std=0.3)
+    yield cfg, weights
+    unregister_architecture("ToyForCausalLM")
+
+
+# ------------------------------------------------- the same model, plainly: whole sequence, no cache
+def plain_toy(weights, ids):
+    w = {k: v.double() for k, v in weights.items()}
+    n = len(ids)
+    cos, sin = (t.double() for t in plain.rope_table(100.0, HD, n))
+
+    def qkv(x, p, kv=True):
+        q = plain.rotate((x @ w[p + ".q_proj.weight"].T).view(n, HEADS, HD), cos, sin)
+        if not kv:
+            return q, None, None
+        k = plain.rotate((x @ w[p + ".k_proj.weight"].T).view(n, KV, HD), cos, sin)
+        return q, k, (x @ w[p + ".v_proj.weight"].T).view(n, KV, HD)
+
+    def attention_layer(s, i, window=None, shared=None):
+        x = plain.rms_norm(s, w[f"l{i}.n1"], 1e-5)
+        q, k, v = qkv(x, f"l{i}.att", kv=shared is None)
+        if shared is not None:
+            k, v = shared
+        o = plain.causal_attention(q, k, v, HD ** -0.5, window).reshape(n, HEADS * HD)
+        s = s + o @ w[f"l{i}.att.o_proj.weight"].T
+        x = plain.rms_norm(s, w[f"l{i}.n2"], 1e-5)
+        s = s + plain.swiglu(x, w[f"l{i}.ff.gate_proj.weight"], w[f"l{i}.ff.up_proj.weight"], w[f"l{i}.ff.down_proj.weight"])
+        return s, (k, v)
+
+    s = w["emb"][torch.tensor(ids)]
+    x = plain.rms_norm(s, w["l0.n1"], 1e-5)
+    state, ys = torch.zeros(WIDTH, dtype=torch.float64), []
+    for t in range(n):
+        state = DECAY * state + x[t]
+        ys.append(state)
+    s = s + torch.stack(ys) @ w["l0.mix.weight"].T
+    x = plain.rms_norm(s, w["l0.n2"], 1e-5)
+    s = s + (torch.tanh(x @ w["l0.ff.a.weight"].T) * (x @ w["l0.ff.b.weight"].T)) @ w["l0.ff.out.weight"].T
+    s, _ = attention_layer(s, 1, window=WINDOW)
+    s, kv2 = attention_layer(s, 2)
+    s, _ = attention_layer(s, 1, window=WINDOW)
+    s, _ = attention_layer(s, 3, shared=kv2)
+    return plain.rms_norm(s, w["out_norm"], 1e-5) @ w["emb"].T
+
+
+LENGTHS = [3, 40, 17, 70, 33]
+
+
+def run_family(toy, family, tmp_path, device, dtype, backend, tol):
+    cfg, weights = toy
+    prompts = trace_util.random_prompts(VOCAB, LENGTHS, seed=21)
+    steps = {"whole": trace_util.whole, "decode_tail": lambda p: trace_util.decode_tail(p, 32),
+             "portions": trace_util.portions, "mixed": lambda p: trace_util.mixed(p, 4, seed=3)}[family](prompts)
+    peak = trace_util.live_token_peak(steps)
+    wts = weights if dtype == "float32" else {k: v.to(torch.bfloat16) for k, v in weights.items()}
+    runner = ModelRunner(cfg, weights=wts, dtype=dtype, device=device, backend=backend, num_pages=peak // 16 + 1,
+                         max_rows=8, max_step_tokens=max(64, peak))
+    assert runner.model.page_groups == [WINDOW, None], "one page group per distinct need"
+    runner.cache.keep_log = True
+    replay(runner, trace_util.to_lines(steps), str(tmp_path), lambda _: None)
+    runner.cache.check()
+    assert not runner.cache.live
+    got = trace_util.read_outputs(str(tmp_path), steps, VOCAB)
+    ref_w = {k: v.float() for k, v in wts.items()}
+    expected = {rid: plain_toy(ref_w, toks) for rid, toks in prompts.items()}
+    worst = trace_util.compare(got, expected, tol, f"toy/{family}/{dtype}")
+    # the windowed group handed pages back while requests were still running
+    assert [p for g, p in runner.cache.released_log if g == 0], "windowed pages must be released"
+    return runner, worst
+
+
+@pytest.mark.parametrize("family", ["whole", "decode_tail", "portions", "mixed"])
+def test_toy_architecture_host(toy, tmp_path, family):
+    runner, _ = run_family(toy, family, tmp_path, "cpu", "float32", TorchBackend(torch.float32), 2e-5)
+    assert runner.num_state_slots == 9
+
+
+def test_window_pages_return_before_the_request_ends(toy):
+    cfg, weights = toy
+    runner = ModelRunner(cfg, weights=weights, dtype="float32", device="cpu", backend=TorchBackend(), num_pages=12,
+                         max_rows=4, max_step_tokens=64)
+    from mini_inference_engine_amd.engine.batch import StepRow
+    rc = runner.cache.open("x")
+    ids = trace_util.random_prompts(VOCAB, [100], seed=1)["r0"]
+    pos = 0
+    for n in (20, 1, 1, 30, 2, 46):
+        assert runner.cache.reserve(rc, pos, n)
+        row = StepRow(rc, ids[pos:pos + n], pos, [n - 1])
+        runner.forward_step([row])
+        runner.after_step([row])
+        pos += n
+        win_pages = [p for p in rc.tables[0] if p]
+        assert len(win_pages) <= WINDOW // 16 + 2, f"{len(win_pages)} window pages held at {pos} tokens"
+        assert len([p for p in rc.tables[1] if p]) == -(-pos // 16)
+    runner.cache.close(rc)
+    runner.cache.check()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("family", ["whole", "decode_tail", "portions", "mixed"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_gpu(toy, tmp_path, family, dtype):
+    run_family(toy, family, tmp_path, "cuda", dtype, None, 2e-5 if dtype == "float32" else 2e-2)
