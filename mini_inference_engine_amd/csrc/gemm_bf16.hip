@@ -4,10 +4,12 @@
 //
 //   y[m, n] = sum_k x[m, k] W[n, k]          W [N, K] bfloat16 as stored in a checkpoint
 //
-// A workgroup of 8 waves owns 16 rows of W (one tile of C^T = W X^T); wave w takes the 32-wide k-steps
-// w, w + 8, ...; v_mfma_f32_16x16x32_bf16 with A = 16 weight rows x 32 k (16 bytes a lane, straight
-// from memory) and B = 32 k x 16 batch rows; the waves' accumulators are summed through LDS in a fixed
-// order.  A row's result depends on nothing but that row, K and the weights: it is bit-identical in any batch.
+// A workgroup of 4 or 8 waves owns 16 rows of W (one tile of C^T = W X^T); each wave streams one
+// contiguous quarter (eighth) of K in 32-wide steps, the loads of the next group of steps in flight while
+// the current group is multiplied; v_mfma_f32_16x16x32_bf16 with A = 16 weight rows x 32 k (16 bytes a
+// lane, straight from memory) and B = 32 k x 16 batch rows; the waves' accumulators are summed through
+// LDS in a fixed order.  A row's result depends on nothing but that row, K, the weights and the number of
+// waves (chosen from N alone): it is bit-identical in any batch.
 //
 // Prologue (NORM): x is not given; instead the 32-bit residual stream r (optionally gathered rows)
 //   and an RMSNorm weight g: x[m, k] = bf16(r[m, k] g[k]), the sum of r^2 is taken on the way, and the
@@ -36,22 +38,24 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 
 enum { EPI_STORE_BF16 = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3 };
 
-#define SG_WAVES 8
-#define SG_THREADS (SG_WAVES * 64)
-
-template <int MT, bool NORM, int EPI>
-__global__ void __launch_bounds__(SG_THREADS)
+template <int MT, bool NORM, int EPI, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
 skinny_gemm_kernel(const void* __restrict__ Xv, long ldx, const int* __restrict__ rows,
                    const void* __restrict__ norm_w, int norm_w_f32, float eps, const bf16* __restrict__ W, long ldw,
                    void* __restrict__ outv, long ldo, int M, int N, int K, int up_offset) {
   constexpr int NT = EPI == EPI_SWIGLU ? 2 : 1;
-  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);        // k-steps in flight per wave
+  constexpr int U = MT == 1 ? (NT == 2 ? 2 : 4) : (MT == 2 ? 2 : 1);     // k-steps per group
+  constexpr int SG_WAVES = WAVES;
+  constexpr int SG_THREADS = WAVES * 64;
   __shared__ float s_acc[SG_WAVES][MT][256];
   __shared__ float s_ss[SG_WAVES][MT * 16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kb = lane >> 4;
   const int n0 = blockIdx.x * 16;
   const int ksteps = (K + 31) >> 5;
+  const int per_wave = (ksteps + SG_WAVES - 1) / SG_WAVES;
+  const int ks0 = wave * per_wave;
+  const int ks1 = ks0 + per_wave < ksteps ? ks0 + per_wave : ksteps;
 
   // weight rows of this lane (clamped for the address; out-of-range rows are zeroed)
   const bf16* wrow[NT];
@@ -82,12 +86,12 @@ skinny_gemm_kernel(const void* __restrict__ Xv, long ldx, const int* __restrict_
     for (int t = 0; t < NT; ++t) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int base = wave; base < ksteps; base += SG_WAVES * U) {
-    Frag a[U][NT], b[U][MT];
+  // one group = U k-steps: the weight fragments a[u][t] and the batch fragments b[u][mt]
+  auto load_group = [&](Frag (&a)[U][NT], Frag (&b)[U][MT], int ks) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int k = (base + SG_WAVES * u) * 32 + kb * 8;
-      const bool kok = k < K;
+      const int k = (ks + u) * 32 + kb * 8;
+      const bool kok = ks + u < ks1 && k < K;
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         a[u][t].q = make_uint4(0, 0, 0, 0);
@@ -132,6 +136,8 @@ skinny_gemm_kernel(const void* __restrict__ Xv, long ldx, const int* __restrict_
         }
       }
     }
+  };
+  auto multiply = [&](Frag (&a)[U][NT], Frag (&b)[U][MT]) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -139,6 +145,15 @@ skinny_gemm_kernel(const void* __restrict__ Xv, long ldx, const int* __restrict_
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
           acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][t].v, b[u][mt].v, acc[t][mt], 0, 0, 0);
+  };
+
+  Frag a0[U][NT], b0[U][MT], a1[U][NT], b1[U][MT];
+  load_group(a0, b0, ks0);
+  for (int ks = ks0; ks < ks1; ks += 2 * U) {
+    load_group(a1, b1, ks + U);          // in flight while group 0 is multiplied
+    multiply(a0, b0);
+    load_group(a0, b0, ks + 2 * U);
+    multiply(a1, b1);
   }
 
   if (NORM) {
@@ -206,12 +221,12 @@ skinny_gemm_kernel(const void* __restrict__ Xv, long ldx, const int* __restrict_
 MIE_EXPORT const char* gemm_bf16_last_error() { return g_mie_error; }
 MIE_EXPORT int mie_skinny_max_rows() { return 64; }
 
-template <int MT, bool NORM>
+template <int MT, bool NORM, int WAVES>
 static int launch_epi(int epi, dim3 grid, hipStream_t s, const void* X, long ldx, const int* rows, const void* norm_w,
                       int norm_w_f32, float eps, const bf16* W, long ldw, void* out, long ldo, int M, int N, int K,
                       int up_offset) {
-#define SG_LAUNCH(E)                                                                                              \
-  hipLaunchKernelGGL((skinny_gemm_kernel<MT, NORM, E>), grid, dim3(SG_THREADS), 0, s, X, ldx, rows, norm_w,       \
+#define SG_LAUNCH(E)                                                                                               \
+  hipLaunchKernelGGL((skinny_gemm_kernel<MT, NORM, E, WAVES>), grid, dim3(WAVES * 64), 0, s, X, ldx, rows, norm_w, \
                      norm_w_f32, eps, W, ldw, out, ldo, M, N, K, up_offset)
   switch (epi) {
     case EPI_STORE_BF16: SG_LAUNCH(EPI_STORE_BF16); break;
@@ -223,6 +238,14 @@ static int launch_epi(int epi, dim3 grid, hipStream_t s, const void* X, long ldx
 #undef SG_LAUNCH
   MIE_CHECK_LAUNCH("skinny_gemm");
   return 0;
+}
+
+template <int MT, bool NORM>
+static int launch_waves(int waves, int epi, dim3 grid, hipStream_t s, const void* X, long ldx, const int* rows,
+                        const void* norm_w, int norm_w_f32, float eps, const bf16* W, long ldw, void* out, long ldo,
+                        int M, int N, int K, int up_offset) {
+  if (waves == 8) return launch_epi<MT, NORM, 8>(epi, grid, s, X, ldx, rows, norm_w, norm_w_f32, eps, W, ldw, out, ldo, M, N, K, up_offset);
+  return launch_epi<MT, NORM, 4>(epi, grid, s, X, ldx, rows, norm_w, norm_w_f32, eps, W, ldw, out, ldo, M, N, K, up_offset);
 }
 
 // X: bfloat16 [M, K] (norm_w null), or the float32 stream with norm_w (RMSNorm weight, bfloat16 or float32)
@@ -242,12 +265,14 @@ MIE_EXPORT int mie_skinny_gemm(const void* X, long ldx, const int* rows, const v
   const int up_offset = N;
   const bf16* Wb = (const bf16*)W;
   const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  // few tiles: more waves per tile, so that enough loads are in flight to fill the memory system
+  const int waves = tiles < 256 ? 8 : 4;
   if (norm_w) {
-    if (MT == 1) return launch_epi<1, true>(epi, grid, s, X, ldx, rows, norm_w, norm_w_f32, eps, Wb, ldw, out, ldo, M, N, K, up_offset);
-    if (MT == 2) return launch_epi<2, true>(epi, grid, s, X, ldx, rows, norm_w, norm_w_f32, eps, Wb, ldw, out, ldo, M, N, K, up_offset);
-    return launch_epi<4, true>(epi, grid, s, X, ldx, rows, norm_w, norm_w_f32, eps, Wb, ldw, out, ldo, M, N, K, up_offset);
+    if (MT == 1) return launch_waves<1, true>(waves, epi, grid, s, X, ldx, rows, norm_w, norm_w_f32, eps, Wb, ldw, out, ldo, M, N, K, up_offset);
+    if (MT == 2) return launch_waves<2, true>(waves, epi, grid, s, X, ldx, rows, norm_w, norm_w_f32, eps, Wb, ldw, out, ldo, M, N, K, up_offset);
+    return launch_waves<4, true>(waves, epi, grid, s, X, ldx, rows, norm_w, norm_w_f32, eps, Wb, ldw, out, ldo, M, N, K, up_offset);
   }
-  if (MT == 1) return launch_epi<1, false>(epi, grid, s, X, ldx, rows, nullptr, 0, 0.f, Wb, ldw, out, ldo, M, N, K, up_offset);
-  if (MT == 2) return launch_epi<2, false>(epi, grid, s, X, ldx, rows, nullptr, 0, 0.f, Wb, ldw, out, ldo, M, N, K, up_offset);
-  return launch_epi<4, false>(epi, grid, s, X, ldx, rows, nullptr, 0, 0.f, Wb, ldw, out, ldo, M, N, K, up_offset);
+  if (MT == 1) return launch_waves<1, false>(waves, epi, grid, s, X, ldx, rows, nullptr, 0, 0.f, Wb, ldw, out, ldo, M, N, K, up_offset);
+  if (MT == 2) return launch_waves<2, false>(waves, epi, grid, s, X, ldx, rows, nullptr, 0, 0.f, Wb, ldw, out, ldo, M, N, K, up_offset);
+  return launch_waves<4, false>(waves, epi, grid, s, X, ldx, rows, nullptr, 0, 0.f, Wb, ldw, out, ldo, M, N, K, up_offset);
 }
