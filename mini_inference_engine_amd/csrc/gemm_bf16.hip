@@ -44,7 +44,8 @@ skinny_gemm_kernel(const void* __restrict__ Xv, long ldx, const int* __restrict_
                    const void* __restrict__ norm_w, int norm_w_f32, float eps, const bf16* __restrict__ W, long ldw,
                    void* __restrict__ outv, long ldo, int M, int N, int K, int up_offset) {
   constexpr int NT = EPI == EPI_SWIGLU ? 2 : 1;
-  constexpr int U = MT == 1 ? (NT == 2 ? 2 : 4) : (MT == 2 ? 2 : 1);     // k-steps per group
+  // k-steps per group of loads; with 8 waves (few tiles) each wave keeps twice as much in flight
+  constexpr int U = (MT == 1 ? (NT == 2 ? 2 : 4) : (MT == 2 ? 2 : 1)) * (WAVES == 8 && !NORM ? 2 : 1);
   constexpr int SG_WAVES = WAVES;
   constexpr int SG_THREADS = WAVES * 64;
   __shared__ float s_acc[SG_WAVES][MT][256];
@@ -86,74 +87,97 @@ skinny_gemm_kernel(const void* __restrict__ Xv, long ldx, const int* __restrict_
     for (int t = 0; t < NT; ++t) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // one group = U k-steps: the weight fragments a[u][t] and the batch fragments b[u][mt]
-  auto load_group = [&](Frag (&a)[U][NT], Frag (&b)[U][MT], int ks) {
+  // One group = U k-steps.  Loads only: nothing here waits for memory, so that the next group's loads
+  // stay in flight while the current group is converted and multiplied.
+  struct Group {
+    Frag a[U][NT];
+    Frag b[U][MT];                 // !NORM: the batch fragments themselves
+    float4 r[NORM ? U : 1][NORM ? MT : 1][2];   // NORM: 8 values of the stream per row and step
+    uint4 g[NORM ? U : 1][2];      // NORM: 8 norm weights per step (bfloat16 in g[.][0], or float32 in both)
+  };
+  auto load_group = [&](Group& G, int ks) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k = (ks + u) * 32 + kb * 8;
       const bool kok = ks + u < ks1 && k < K;
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        a[u][t].q = make_uint4(0, 0, 0, 0);
-        if (kok && wok[t]) a[u][t].q = *reinterpret_cast<const uint4*>(wrow[t] + k);
+        G.a[u][t].q = make_uint4(0, 0, 0, 0);
+        if (kok && wok[t]) G.a[u][t].q = *reinterpret_cast<const uint4*>(wrow[t] + k);
       }
       if (NORM) {
-        float g[8];
+        G.g[u][0] = make_uint4(0, 0, 0, 0);
+        G.g[u][1] = make_uint4(0, 0, 0, 0);
         if (kok) {
           if (norm_w_f32) {
-            const float4 g0 = *reinterpret_cast<const float4*>((const float*)norm_w + k);
-            const float4 g1 = *reinterpret_cast<const float4*>((const float*)norm_w + k + 4);
-            g[0] = g0.x; g[1] = g0.y; g[2] = g0.z; g[3] = g0.w; g[4] = g1.x; g[5] = g1.y; g[6] = g1.z; g[7] = g1.w;
+            G.g[u][0] = *reinterpret_cast<const uint4*>((const float*)norm_w + k);
+            G.g[u][1] = *reinterpret_cast<const uint4*>((const float*)norm_w + k + 4);
           } else {
-            const uint4 gw = *reinterpret_cast<const uint4*>((const bf16*)norm_w + k);
-            const uint32_t w4[4] = {gw.x, gw.y, gw.z, gw.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              g[2 * j] = __uint_as_float(w4[j] << 16);
-              g[2 * j + 1] = __uint_as_float(w4[j] & 0xFFFF0000u);
-            }
+            G.g[u][0] = *reinterpret_cast<const uint4*>((const bf16*)norm_w + k);
           }
         }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          b[u][mt].q = make_uint4(0, 0, 0, 0);
+          G.r[u][mt][0] = make_float4(0.f, 0.f, 0.f, 0.f);
+          G.r[u][mt][1] = make_float4(0.f, 0.f, 0.f, 0.f);
           if (kok && xok[mt]) {
             const float* rp = (const float*)xrow[mt] + k;
-            const float4 r0 = *reinterpret_cast<const float4*>(rp);
-            const float4 r1 = *reinterpret_cast<const float4*>(rp + 4);
-            const float r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
-#pragma unroll
-            for (int j = 0; j < 8; ++j) ss[mt] = fmaf(r[j], r[j], ss[mt]);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) b[u][mt].w[j] = pack_bf16(r[2 * j] * g[2 * j], r[2 * j + 1] * g[2 * j + 1]);
+            G.r[u][mt][0] = *reinterpret_cast<const float4*>(rp);
+            G.r[u][mt][1] = *reinterpret_cast<const float4*>(rp + 4);
           }
         }
       } else {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          b[u][mt].q = make_uint4(0, 0, 0, 0);
-          if (kok && xok[mt]) b[u][mt].q = *reinterpret_cast<const uint4*>((const bf16*)xrow[mt] + k);
+          G.b[u][mt].q = make_uint4(0, 0, 0, 0);
+          if (kok && xok[mt]) G.b[u][mt].q = *reinterpret_cast<const uint4*>((const bf16*)xrow[mt] + k);
         }
       }
     }
   };
-  auto multiply = [&](Frag (&a)[U][NT], Frag (&b)[U][MT]) {
+  auto multiply = [&](Group& G) {
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
+      if (NORM) {
+        float g[8];
+        if (norm_w_f32) {
+          const uint32_t w8[8] = {G.g[u][0].x, G.g[u][0].y, G.g[u][0].z, G.g[u][0].w,
+                                  G.g[u][1].x, G.g[u][1].y, G.g[u][1].z, G.g[u][1].w};
+#pragma unroll
+          for (int j = 0; j < 8; ++j) g[j] = __uint_as_float(w8[j]);
+        } else {
+          const uint32_t w4[4] = {G.g[u][0].x, G.g[u][0].y, G.g[u][0].z, G.g[u][0].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            g[2 * j] = __uint_as_float(w4[j] << 16);
+            g[2 * j + 1] = __uint_as_float(w4[j] & 0xFFFF0000u);
+          }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const float4 r0 = G.r[u][mt][0], r1 = G.r[u][mt][1];
+          const float r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+#pragma unroll
+          for (int j = 0; j < 8; ++j) ss[mt] = fmaf(r[j], r[j], ss[mt]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) G.b[u][mt].w[j] = pack_bf16(r[2 * j] * g[2 * j], r[2 * j + 1] * g[2 * j + 1]);
+        }
+      }
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][t].v, b[u][mt].v, acc[t][mt], 0, 0, 0);
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(G.a[u][t].v, G.b[u][mt].v, acc[t][mt], 0, 0, 0);
+    }
   };
 
-  Frag a0[U][NT], b0[U][MT], a1[U][NT], b1[U][MT];
-  load_group(a0, b0, ks0);
+  Group g0, g1;
+  load_group(g0, ks0);
   for (int ks = ks0; ks < ks1; ks += 2 * U) {
-    load_group(a1, b1, ks + U);          // in flight while group 0 is multiplied
-    multiply(a0, b0);
-    load_group(a0, b0, ks + 2 * U);
-    multiply(a1, b1);
+    load_group(g1, ks + U);          // in flight while group 0 is multiplied
+    multiply(g0);
+    load_group(g0, ks + 2 * U);
+    multiply(g1);
   }
 
   if (NORM) {
