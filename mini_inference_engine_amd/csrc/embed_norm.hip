@@ -65,6 +65,74 @@ add_rmsnorm_kernel(const TX* __restrict__ x, float* __restrict__ stream, const T
   }
 }
 
+
+// Few rows (a decode step): the whole cost is latency, so every load of a row (stream, pending x and
+// weight) is issued before anything is reduced, 4 elements a lane at a time.  Same arithmetic and the
+// same order of the block reduction inputs as above is not required: the fast path is taken for a row
+// whenever width % 4 == 0 and width <= 4 * NORM_FAST_THREADS * NORM_FAST_VEC, whatever the batch is,
+// so a row's result still does not depend on the batch.
+#define NORM_FAST_THREADS 256
+#define NORM_FAST_VEC 8      // float4 groups per thread: widths up to 8192
+
+template <typename T> __device__ __forceinline__ float4 load4(const T* p);
+template <> __device__ __forceinline__ float4 load4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 load4<bf16>(const bf16* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xFFFF0000u), __uint_as_float(u.y << 16),
+                     __uint_as_float(u.y & 0xFFFF0000u));
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16* p, float4 v) {
+  uint2 u;
+  u.x = (uint32_t)__bfloat16_as_ushort(__float2bfloat16(v.x)) | ((uint32_t)__bfloat16_as_ushort(__float2bfloat16(v.y)) << 16);
+  u.y = (uint32_t)__bfloat16_as_ushort(__float2bfloat16(v.z)) | ((uint32_t)__bfloat16_as_ushort(__float2bfloat16(v.w)) << 16);
+  *reinterpret_cast<uint2*>(p) = u;
+}
+
+template <typename TX, typename TW, typename TY>
+__global__ void __launch_bounds__(NORM_FAST_THREADS)
+add_rmsnorm_fast_kernel(const TX* __restrict__ x, float* __restrict__ stream, const TW* __restrict__ weight,
+                        TY* __restrict__ y, const int* __restrict__ rows, int width, float eps) {
+  __shared__ float scratch[16];
+  const int out_row = blockIdx.x;
+  const int row = rows ? rows[out_row] : out_row;
+  float* sr = stream + (size_t)row * width;
+  const TX* xr = x ? x + (size_t)row * width : nullptr;
+  float4 r[NORM_FAST_VEC], w[NORM_FAST_VEC];
+#pragma unroll
+  for (int k = 0; k < NORM_FAST_VEC; ++k) {
+    const int i = (threadIdx.x + k * NORM_FAST_THREADS) * 4;
+    r[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    w[k] = r[k];
+    if (i < width) {
+      r[k] = load4(sr + i);
+      w[k] = load4(weight + i);
+      if (xr) {
+        const float4 a = load4(xr + i);
+        r[k].x += a.x; r[k].y += a.y; r[k].z += a.z; r[k].w += a.w;
+      }
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NORM_FAST_VEC; ++k) {
+    ss = fmaf(r[k].x, r[k].x, ss); ss = fmaf(r[k].y, r[k].y, ss);
+    ss = fmaf(r[k].z, r[k].z, ss); ss = fmaf(r[k].w, r[k].w, ss);
+    const int i = (threadIdx.x + k * NORM_FAST_THREADS) * 4;
+    if (xr && !rows && i < width) store4(sr + i, r[k]);
+  }
+  const float total = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(total / (float)width + eps);
+  TY* yr = y + (size_t)out_row * width;
+#pragma unroll
+  for (int k = 0; k < NORM_FAST_VEC; ++k) {
+    const int i = (threadIdx.x + k * NORM_FAST_THREADS) * 4;
+    if (i < width)
+      store4(yr + i, make_float4(r[k].x * rstd * w[k].x, r[k].y * rstd * w[k].y, r[k].z * rstd * w[k].z,
+                                 r[k].w * rstd * w[k].w));
+  }
+}
+
 MIE_EXPORT const char* embed_norm_last_error() { return g_mie_error; }
 
 MIE_EXPORT int mie_embedding(const int* ids, const void* table, int table_dtype, float* out, int tokens, int width,
@@ -86,14 +154,22 @@ template <typename TX, typename TW>
 static int launch_norm(const void* x, float* stream, const void* w, void* y, int y_dtype, const int* rows, int n_rows,
                        int width, float eps, hipStream_t s) {
   dim3 grid(n_rows), block(NORM_THREADS);
-  if (y_dtype == MIE_F32)
+  // the vector kernel whenever the width allows it (a property of the model, not of the batch)
+  const bool fast = width % 4 == 0 && width <= 4 * NORM_FAST_THREADS * NORM_FAST_VEC &&
+                    (((uintptr_t)x | (uintptr_t)stream | (uintptr_t)w | (uintptr_t)y) & 15) == 0;
+  if (y_dtype != MIE_F32 && y_dtype != MIE_BF16) MIE_FAIL("add_rmsnorm: output dtype code %d", y_dtype);
+  if (fast && y_dtype == MIE_F32)
+    hipLaunchKernelGGL((add_rmsnorm_fast_kernel<TX, TW, float>), grid, dim3(NORM_FAST_THREADS), 0, s, (const TX*)x,
+                       stream, (const TW*)w, (float*)y, rows, width, eps);
+  else if (fast)
+    hipLaunchKernelGGL((add_rmsnorm_fast_kernel<TX, TW, bf16>), grid, dim3(NORM_FAST_THREADS), 0, s, (const TX*)x,
+                       stream, (const TW*)w, (bf16*)y, rows, width, eps);
+  else if (y_dtype == MIE_F32)
     hipLaunchKernelGGL((add_rmsnorm_kernel<TX, TW, float>), grid, block, 0, s, (const TX*)x, stream, (const TW*)w,
                        (float*)y, rows, width, eps);
-  else if (y_dtype == MIE_BF16)
+  else
     hipLaunchKernelGGL((add_rmsnorm_kernel<TX, TW, bf16>), grid, block, 0, s, (const TX*)x, stream, (const TW*)w,
                        (bf16*)y, rows, width, eps);
-  else
-    MIE_FAIL("add_rmsnorm: output dtype code %d", y_dtype);
   MIE_CHECK_LAUNCH("add_rmsnorm");
   return 0;
 }

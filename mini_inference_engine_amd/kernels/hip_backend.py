@@ -87,8 +87,8 @@ class HipBackend(KernelBackend):
                 "mie_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
             },
             "gemm_bf16": {
-                "mie_skinny_gemm": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_long, c_void_p,
-                                    c_long, c_int, c_int, c_int, c_int, c_void_p],
+                "mie_skinny_gemm": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_int,
+                                    c_void_p],
                 "mie_skinny_max_rows": [],
             },
             "attention_bf16": {
@@ -168,27 +168,15 @@ class HipBackend(KernelBackend):
     EPI_BF16, EPI_F32, EPI_ADD, EPI_SWIGLU = 0, 1, 2, 3
 
     def _skinny_ok(self, x, w, bias) -> bool:
-        rows = x.shape[0]
-        src = x.residual if isinstance(x, Normed) else x
-        return (not self.true_fp32 and bias is None and w.dtype == torch.bfloat16 and rows <= self.SKINNY_MAX_ROWS
-                and w.shape[1] % 8 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
-                and src.data_ptr() % 16 == 0 and src.stride(0) % 8 == 0
-                and (isinstance(x, Normed) or x.dtype == torch.bfloat16)
-                and (not isinstance(x, Normed) or (x.pending is None and x._value is None
-                                                   and x.weight.data_ptr() % 16 == 0)))
+        """Whether the fused few-row kernel takes this product (x a bfloat16 tensor)."""
+        return (not self.true_fp32 and bias is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+                and x.shape[0] <= self.SKINNY_MAX_ROWS and w.shape[1] % 8 == 0 and w.stride(0) % 8 == 0
+                and x.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0)
 
     def _skinny(self, x, w, epi, out, n_out):
         lib = self.lib("gemm_bf16")
-        if isinstance(x, Normed):
-            src, rows, nw = x.residual, x.rows, x.weight
-            M = src.shape[0] if rows is None else rows.shape[0]
-            library.check(lib, lib.mie_skinny_gemm(
-                _ptr(src), src.stride(0), _ptr(rows), _ptr(nw), int(nw.dtype == torch.float32), float(x.eps),
-                _ptr(w), w.stride(0), _ptr(out), out.stride(0), epi, M, n_out, w.shape[1], self._stream()))
-        else:
-            library.check(lib, lib.mie_skinny_gemm(
-                _ptr(x), x.stride(0), None, None, 0, 0.0, _ptr(w), w.stride(0), _ptr(out), out.stride(0), epi,
-                x.shape[0], n_out, w.shape[1], self._stream()))
+        library.check(lib, lib.mie_skinny_gemm(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), epi,
+                                               x.shape[0], n_out, w.shape[1], self._stream()))
         return out
 
     def linear(self, x, w, bias=None, out_dtype=None, add_to=None):
@@ -202,16 +190,16 @@ class HipBackend(KernelBackend):
         if add_to is not None and (add_to.dtype != torch.float32 or tuple(add_to.shape) != (M, N)
                                    or not add_to.is_contiguous()):
             raise ValueError(f"linear: add_to must be the contiguous float32 stream {(M, N)}")
+        if isinstance(x, Normed):
+            x = x.materialize()
+        self._on_device(x)
+        _rows_ok(x, "linear: x")
         if self._skinny_ok(x, w, bias) and out_dtype in (torch.bfloat16, torch.float32):
             if add_to is not None:
                 self._skinny(x, w, self.EPI_ADD, add_to, N)
                 return None
             out = torch.empty((M, N), dtype=out_dtype, device=w.device)
             return self._skinny(x, w, self.EPI_BF16 if out_dtype == torch.bfloat16 else self.EPI_F32, out, N)
-        if isinstance(x, Normed):
-            x = x.materialize()
-        self._on_device(x)
-        _rows_ok(x, "linear: x")
         if not self.true_fp32 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
             # library matrix product, 32-bit accumulation, as the reference's F.linear
             y = torch.nn.functional.linear(x, w, None if bias is None else bias.to(torch.bfloat16))
@@ -233,6 +221,8 @@ class HipBackend(KernelBackend):
             raise ValueError(f"linear_silu_mul: weight of {w_gate_up.shape[0]} rows for intermediate {intermediate}")
         if x.shape[1] != w_gate_up.shape[1]:
             raise ValueError(f"linear_silu_mul: x {tuple(x.shape)} against w {tuple(w_gate_up.shape)}")
+        if isinstance(x, Normed):
+            x = x.materialize()
         if self._skinny_ok(x, w_gate_up, None):
             out = torch.empty((x.shape[0], intermediate), dtype=torch.bfloat16, device=w_gate_up.device)
             return self._skinny(x, w_gate_up, self.EPI_SWIGLU, out, intermediate)
