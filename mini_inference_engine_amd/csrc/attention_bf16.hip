@@ -10,8 +10,8 @@
 // taken in the order (lane group, tile, i), and the value operand is loaded in that same order, so the
 // probabilities never leave registers.  Softmax state (max, sum) is one value per lane (its head);
 // exponentials are base 2 with scale * log2(e) folded into the scores.  The waves of a workgroup are
-// merged through LDS; splits write normalised partials and base-2 log-sum-exps, and the split that
-// arrives last (an atomic counter per row and head tile) merges them.  Keys outside [lo, p] get probability 0 by selection and their values are zeroed, so stale
+// merged through LDS; splits write normalised partials and base-2 log-sum-exps, merged by a second
+// kernel.  Keys outside [lo, p] get probability 0 by selection and their values are zeroed, so stale
 // or poisoned slots never reach the sums.
 #include "common.hpp"
 
@@ -51,10 +51,9 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
                         const bf16* __restrict__ v_cache, bf16* __restrict__ out, float* __restrict__ o_part,
                         float* __restrict__ lse_part, const int* __restrict__ block_tables, int max_blocks,
                         const int* __restrict__ positions, int Hq, int Hkv, int head_tiles, int page,
-                        float scale_log2, int window, int partition, int num_splits, int* __restrict__ arrivals) {
+                        float scale_log2, int window, int partition, int num_splits) {
   __shared__ float s_m[NW][16], s_l[NW][16], s_M[16], s_L[16];
   __shared__ float s_o[NW][16][D + 1];
-  __shared__ int s_last;
   const int b = blockIdx.x;
   const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
   const int s = blockIdx.z;
@@ -69,7 +68,11 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
   const bool head_ok = g < G;
   const int head = kvh * G + (head_ok ? g : 0);
 
-  const bool empty = begin > pos;      // this split lies beyond the row's keys (uniform over the workgroup)
+  if (begin > pos) {          // this split lies beyond the row's keys (uniform over the workgroup)
+    if (num_splits > 1 && threadIdx.x < 16 && ht * 16 + (int)threadIdx.x < G)
+      lse_part[((size_t)b * Hq + kvh * G + ht * 16 + threadIdx.x) * num_splits + s] = -INFINITY;
+    return;
+  }
 
   const int* bt = block_tables + (size_t)b * max_blocks;
   Frag qf[KS];
@@ -85,7 +88,7 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) O[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int blk = begin + BLOCK_KEYS * wave; blk < end && !empty; blk += BLOCK_KEYS * NW) {
+  for (int blk = begin + BLOCK_KEYS * wave; blk < end; blk += BLOCK_KEYS * NW) {
     // ---- scores of 32 keys x 16 heads
     f32x4 S[2];
 #pragma unroll
@@ -200,15 +203,11 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
     const int hc = e / D, d = e - hc * D;
     const int gg = ht * 16 + hc;
     if (gg >= G) continue;
-    const size_t hh = (size_t)b * Hq + kvh * G + gg;
-    if (empty) {
-      if (d == 0) lse_part[hh * num_splits + s] = -INFINITY;
-      continue;
-    }
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) sum += s_o[w][hc][d];
     const float val = sum / s_L[hc];
+    const size_t hh = (size_t)b * Hq + kvh * G + gg;
     if (num_splits == 1) {
       out[hh * D + d] = __float2bfloat16(val);
     } else {
@@ -216,46 +215,25 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
       if (d == 0) lse_part[hh * num_splits + s] = s_M[hc] + log2f(s_L[hc]);
     }
   }
-  if (num_splits == 1) return;
+}
 
-  // ---- the split that arrives last merges all of them (no second kernel)
-  __threadfence();                       // this workgroup's partials are visible before it is counted
-  __syncthreads();
-  int* counter = arrivals + (size_t)b * gridDim.y + blockIdx.y;
-  if (threadIdx.x == 0) {
-    const int before = atomicAdd(counter, 1);
-    s_last = before == num_splits - 1;
-    if (s_last) *counter = 0;            // left at zero for the next call
-  }
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();                       // see the other workgroups' partials
-  if (threadIdx.x < 16) {
-    const int gg = ht * 16 + threadIdx.x;
-    float M2 = -INFINITY, W2 = 0.f;
-    if (gg < G) {
-      const float* lse = lse_part + ((size_t)b * Hq + kvh * G + gg) * num_splits;
-      for (int i = 0; i < num_splits; ++i) M2 = fmaxf(M2, lse[i]);
-      for (int i = 0; i < num_splits; ++i) W2 += lse[i] == -INFINITY ? 0.f : exp2f(lse[i] - M2);
-    }
-    s_M[threadIdx.x] = M2;
-    s_L[threadIdx.x] = W2;
-  }
-  __syncthreads();
-  for (int e = threadIdx.x; e < 16 * D; e += NW * 64) {
-    const int hc = e / D, d = e - hc * D;
-    const int gg = ht * 16 + hc;
-    if (gg >= G) continue;
-    const size_t hh = (size_t)b * Hq + kvh * G + gg;
-    const float* lse = lse_part + hh * num_splits;
-    const float* op = o_part + hh * num_splits * D + d;
-    const float M2 = s_M[hc];
+__global__ void __launch_bounds__(64)
+merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ lse_part, bf16* __restrict__ out,
+                    int num_splits) {
+  const size_t hh = blockIdx.x;
+  const float* lse = lse_part + hh * num_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, lse[s]);
+  float W = 0.f;
+  for (int s = 0; s < num_splits; ++s) W += lse[s] == -INFINITY ? 0.f : exp2f(lse[s] - M);
+  const float inv = 1.0f / W;
+  for (int d = threadIdx.x; d < D; d += 64) {
     float acc = 0.f;
-    for (int i = 0; i < num_splits; ++i) {
-      const float ls = lse[i];
-      if (ls != -INFINITY) acc += exp2f(ls - M2) * op[(size_t)i * D];
+    for (int s = 0; s < num_splits; ++s) {
+      const float ls = lse[s];
+      if (ls != -INFINITY) acc += exp2f(ls - M) * o_part[(hh * num_splits + s) * D + d];
     }
-    out[hh * D + d] = __float2bfloat16(acc / s_L[hc]);
+    out[hh * D + d] = __float2bfloat16(acc * inv);
   }
 }
 
@@ -444,21 +422,19 @@ MIE_EXPORT int mie_attention_bf16_head_dim() { return D; }
 MIE_EXPORT int mie_decode_block_keys() { return BLOCK_KEYS * NW; }
 
 // q: token b is row b (single-token rows lead the flattened batch).  partition: keys per split, a
-// multiple of mie_decode_block_keys().  When num_splits > 1: o_part [rows, Hq, splits, D] and
-// lse_part [rows, Hq, splits] float, and arrivals, int32 [rows * Hkv * ceil(group / 16)] that must be zero
-// before the first call and is left zero by every call (calls that share it must not overlap).
+// multiple of mie_decode_block_keys().  o_part [rows, Hq, splits, D] and lse_part [rows, Hq, splits]
+// float are needed when num_splits > 1.
 MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
-                                    float* o_part, float* lse_part, int* arrivals, const int* block_tables,
-                                    int max_blocks, const int* positions, int rows, int Hq, int Hkv, int head_dim,
-                                    int page, float scale, int window, int partition, int num_splits,
-                                    hipStream_t stream) {
+                                    float* o_part, float* lse_part, const int* block_tables, int max_blocks,
+                                    const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
+                                    float scale, int window, int partition, int num_splits, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (head_dim != D) MIE_FAIL("decode_attention: built for head_dim %d, called with %d", D, head_dim);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("decode_attention: %d query heads on %d kv heads", Hq, Hkv);
   if (page < 16 || page % 16) MIE_FAIL("decode_attention: page size %d (multiples of 16)", page);
   if (partition <= 0 || partition % (BLOCK_KEYS * NW)) MIE_FAIL("decode_attention: partition %d is no multiple of %d", partition, BLOCK_KEYS * NW);
   if (num_splits < 1 || num_splits > 65535) MIE_FAIL("decode_attention: %d splits", num_splits);
-  if (num_splits > 1 && (!o_part || !lse_part || !arrivals)) MIE_FAIL("decode_attention: splits need partial buffers and arrival counters");
+  if (num_splits > 1 && (!o_part || !lse_part)) MIE_FAIL("decode_attention: splits need partial buffers");
   if (q_stride < (long)Hq * D || (q_stride % 8) || ((uintptr_t)q % 16)) MIE_FAIL("decode_attention: q stride %ld / alignment", q_stride);
   if (max_blocks <= 0) MIE_FAIL("decode_attention: max_blocks %d", max_blocks);
   const int G = Hq / Hkv, head_tiles = (G + 15) / 16;
@@ -466,8 +442,12 @@ MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_
   dim3 grid(rows, Hkv * head_tiles, num_splits), block(NW * 64);
   hipLaunchKernelGGL(decode_attention_kernel, grid, block, 0, stream, (const bf16*)q, q_stride, (const bf16*)k_cache,
                      (const bf16*)v_cache, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv,
-                     head_tiles, page, scale * 1.4426950408889634f, window, partition, num_splits, arrivals);
+                     head_tiles, page, scale * 1.4426950408889634f, window, partition, num_splits);
   MIE_CHECK_LAUNCH("decode_attention");
+  if (num_splits > 1) {
+    hipLaunchKernelGGL(merge_splits_kernel, dim3(rows * Hq), dim3(64), 0, stream, o_part, lse_part, (bf16*)out, num_splits);
+    MIE_CHECK_LAUNCH("merge_splits");
+  }
   return 0;
 }
 

@@ -93,8 +93,8 @@ class HipBackend(KernelBackend):
             },
             "attention_bf16": {
                 "mie_decode_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                         c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                         c_int, c_int, c_void_p],
+                                         c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                         c_int, c_void_p],
                 "mie_prefill_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                           c_void_p],
@@ -285,16 +285,6 @@ class HipBackend(KernelBackend):
     # workgroups the decode attention kernel should at least be spread over (two per compute unit)
     DECODE_TARGET_WORKGROUPS = 512
 
-    def _arrival_counters(self, n: int):
-        """Zeroed int32 counters for the decode kernel's split merge.  One buffer per backend: every call
-        leaves it zero, and calls on one stream do not overlap.  It only ever grows (outside graph capture)."""
-        have = getattr(self, "_arrivals", None)
-        if have is None or have.numel() < n:
-            if torch.cuda.is_current_stream_capturing():
-                raise RuntimeError("decode attention needs more arrival counters than were made before capture")
-            self._arrivals = torch.zeros(max(n, 4096), dtype=torch.int32, device=self.device)
-        return self._arrivals
-
     def decode_splits(self, rows: int, Hq: int, Hkv: int, context_bound: int, window, block_keys: int):
         """(keys per split, number of splits) for single-token rows: split the context only as far
         as the rows and heads alone do not fill the GPU (inference_engine/kernels/decode_attention.py:117-125
@@ -323,15 +313,14 @@ class HipBackend(KernelBackend):
                 bound = min(step.max_context, window + 32) if window else step.max_context
                 partition = -(-(-(-bound // num_splits)) // block_keys) * block_keys
                 splits = max(1, -(-bound // partition))
-            o_part = lse_part = arrivals = None
+            o_part = lse_part = None
             if splits > 1:
                 o_part = torch.empty((done, Hq, splits, D), dtype=torch.float32, device=qkv.device)
                 lse_part = torch.empty((done, Hq, splits), dtype=torch.float32, device=qkv.device)
-                arrivals = self._arrival_counters(done * Hkv * -(-(Hq // Hkv) // 16))
             library.check(lib, lib.mie_decode_attention(
                 _ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(o_part), _ptr(lse_part),
-                _ptr(arrivals), _ptr(bt), bt.shape[1], _ptr(step.positions), done, Hq, Hkv, D, page, float(scale),
-                int(window or 0), partition, splits, self._stream()))
+                _ptr(bt), bt.shape[1], _ptr(step.positions), done, Hq, Hkv, D, page, float(scale), int(window or 0),
+                partition, splits, self._stream()))
         if done < T and qkv.dtype == torch.bfloat16 and not force_generic:
             # rows of several tokens: matrix-core kernel over their own and earlier portions' keys
             for name, t, n in (("row_start", step.row_start, step.num_rows + 1),
