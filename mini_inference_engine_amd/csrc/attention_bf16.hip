@@ -10,8 +10,8 @@
 // taken in the order (lane group, tile, i), and the value operand is loaded in that same order, so the
 // probabilities never leave registers.  Softmax state (max, sum) is one value per lane (its head);
 // exponentials are base 2 with scale * log2(e) folded into the scores.  The waves of a workgroup are
-// merged through LDS; splits write normalised partials and base-2 log-sum-exps, merged by a second
-// kernel.  Keys outside [lo, p] get probability 0 by selection and their values are zeroed, so stale
+// merged through LDS; splits write normalised partials and base-2 log-sum-exps, merged by a second,
+// small kernel.  Keys outside [lo, p] get probability 0 by selection and their values are zeroed, so stale
 // or poisoned slots never reach the sums.
 #include "common.hpp"
 
@@ -217,26 +217,58 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
   }
 }
 
+// One wave per (row, head): lane s takes the log-sum-exp of split s (the wave reduces max and sum with
+// shuffles), then the lanes spread over D and add the splits' partials with all loads of a chunk of 16
+// splits issued together: two memory round trips in all, whatever the number of splits.
+// (Merging inside the attention kernel by the split that arrives last was tried: the partials have to
+// cross the per-XCD L2s, and the device-scope fences that takes cost far more than this launch.)
 __global__ void __launch_bounds__(64)
 merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ lse_part, bf16* __restrict__ out,
                     int num_splits) {
+  constexpr int DL = (D + 63) / 64;
   const size_t hh = blockIdx.x;
+  const int lane = threadIdx.x;
   const float* lse = lse_part + hh * num_splits;
-  float M = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, lse[s]);
+  const float* op = o_part + hh * num_splits * D;
+  float acc[DL];
+#pragma unroll
+  for (int i = 0; i < DL; ++i) acc[i] = 0.f;
   float W = 0.f;
-  for (int s = 0; s < num_splits; ++s) W += lse[s] == -INFINITY ? 0.f : exp2f(lse[s] - M);
-  const float inv = 1.0f / W;
-  for (int d = threadIdx.x; d < D; d += 64) {
-    float acc = 0.f;
-    for (int s = 0; s < num_splits; ++s) {
-      const float ls = lse[s];
-      if (ls != -INFINITY) acc += exp2f(ls - M) * o_part[(hh * num_splits + s) * D + d];
+  float M = -INFINITY;                       // the maximum over all splits first (64 a round)
+  for (int s0 = 0; s0 < num_splits; s0 += 64) {
+    const float v = s0 + lane < num_splits ? lse[s0 + lane] : -INFINITY;
+    M = fmaxf(M, wave_max(v));
+  }
+  for (int s0 = 0; s0 < num_splits; s0 += 64) {
+    const float v = s0 + lane < num_splits ? lse[s0 + lane] : -INFINITY;
+    const float w = v == -INFINITY ? 0.f : exp2f(v - M);
+    W += wave_sum(w);
+    const int n = num_splits - s0 < 64 ? num_splits - s0 : 64;
+    for (int c = 0; c < n; c += 16) {
+      float part[16][DL];
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+#pragma unroll
+        for (int i = 0; i < DL; ++i) {
+          const int d = lane + 64 * i;
+          part[j][i] = (c + j < n && d < D) ? op[(size_t)(s0 + c + j) * D + d] : 0.f;
+        }
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const float wj = __shfl(w, (c + j) & 63, 64);
+#pragma unroll
+        for (int i = 0; i < DL; ++i)
+          if (c + j < n && wj != 0.f) acc[i] += wj * part[j][i];    // a split without keys holds no data
+      }
     }
-    out[hh * D + d] = __float2bfloat16(acc * inv);
+  }
+  const float inv = 1.0f / W;
+#pragma unroll
+  for (int i = 0; i < DL; ++i) {
+    const int d = lane + 64 * i;
+    if (d < D) out[hh * D + d] = __float2bfloat16(acc[i] * inv);
   }
 }
-
 
 // prefill_attention: rows of several tokens, starting anywhere in their request.  The same two
 // products as above with "head" replaced by "query": S^T[key, query] = K . Q^T and
