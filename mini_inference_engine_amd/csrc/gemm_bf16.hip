@@ -34,13 +34,25 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return (ua >> 16) | (ub & 0xFFFF0000u);
 }
 
-enum { EPI_STORE_BF16 = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3 };
+enum { EPI_STORE_BF16 = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3, EPI_ROPE = 4 };
+
+// What the rotary epilogue needs beside the product: W is the fused q/k/v projection; the workgroup owns
+// columns j0 .. j0 + 15 and j0 + D/2 .. j0 + D/2 + 15 of one head, i.e. 16 rotary pairs.
+struct RopeArgs {
+  const int* positions;      // [M]
+  const float* cos_t;        // [positions, D / 2]
+  const float* sin_t;
+  const int* slots;          // [M] cache slot of each row's token
+  bf16* k_cache;             // [pages, Hkv, page, D]
+  bf16* v_cache;             // [pages, Hkv, D, page]
+  int Hq, Hkv, D, page;
+};
 
 template <int MT, int EPI, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
 skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict__ W, long ldw, void* __restrict__ outv,
-                   long ldo, int M, int N, int K, int up_offset) {
-  constexpr int NT = EPI == EPI_SWIGLU ? 2 : 1;
+                   long ldo, int M, int N, int K, int up_offset, RopeArgs rope) {
+  constexpr int NT = (EPI == EPI_SWIGLU || EPI == EPI_ROPE) ? 2 : 1;
   // k-steps per group of loads (two groups are in flight per wave)
 #ifndef SG_U_SCALE
 #define SG_U_SCALE 1
@@ -51,7 +63,11 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
   __shared__ float s_acc[SG_WAVES][MT][256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kb = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  int n0 = blockIdx.x * 16;
+  if (EPI == EPI_ROPE) {                     // tiles are numbered per head: D / 32 pairs of tiles each
+    const int per_head = rope.D >> 5;
+    n0 = (blockIdx.x / per_head) * rope.D + (blockIdx.x % per_head) * 16;
+  }
   const int ksteps = (K + 31) >> 5;
   const int per_wave = (ksteps + SG_WAVES - 1) / SG_WAVES;
   const int ks0 = wave * per_wave;
@@ -164,7 +180,33 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
     const int m = e >> 4, n = n0 + (e & 15);
     if (m >= M || n >= N) continue;
     const size_t o = (size_t)m * ldo + n;
-    if (EPI == EPI_STORE_BF16) {
+    if (EPI == EPI_ROPE) {
+      const int D = rope.D, half = D >> 1;
+      const int head = n / D, jd = n - head * D;         // jd < D / 2: the first of the pair
+      const float x1 = v[0][j], x2 = v[NT - 1][j];
+      if (head < rope.Hq + rope.Hkv) {
+        const int pos = rope.positions[m];
+        const float c = rope.cos_t[(size_t)pos * half + jd], sn = rope.sin_t[(size_t)pos * half + jd];
+        const bf16 o1 = __float2bfloat16(x1 * c - x2 * sn), o2 = __float2bfloat16(x2 * c + x1 * sn);
+        if (head < rope.Hq) {
+          bf16* q = (bf16*)outv + (size_t)m * ldo + (size_t)head * D + jd;
+          q[0] = o1;
+          q[half] = o2;
+        } else {
+          const int slot = rope.slots[m];
+          bf16* kc = rope.k_cache + (((size_t)(slot / rope.page) * rope.Hkv + (head - rope.Hq)) * rope.page +
+                                     slot % rope.page) * D + jd;
+          kc[0] = o1;
+          kc[half] = o2;
+        }
+      } else {
+        const int slot = rope.slots[m];
+        bf16* vc = rope.v_cache + (((size_t)(slot / rope.page) * rope.Hkv + (head - rope.Hq - rope.Hkv)) * D + jd) *
+                                      rope.page + slot % rope.page;
+        vc[0] = __float2bfloat16(x1);
+        vc[(size_t)half * rope.page] = __float2bfloat16(x2);
+      }
+    } else if (EPI == EPI_STORE_BF16) {
       ((bf16*)outv)[o] = __float2bfloat16(v[0][j]);
     } else if (EPI == EPI_STORE_F32) {
       ((float*)outv)[o] = v[0][j];
@@ -182,15 +224,16 @@ MIE_EXPORT int mie_skinny_max_rows() { return 64; }
 
 template <int MT, int WAVES>
 static int launch_epi(int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx, const bf16* W, long ldw, void* out,
-                      long ldo, int M, int N, int K, int up_offset) {
+                      long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope) {
 #define SG_LAUNCH(E)                                                                                           \
   hipLaunchKernelGGL((skinny_gemm_kernel<MT, E, WAVES>), grid, dim3(WAVES * 64), 0, s, X, ldx, W, ldw, out, ldo, M, N, \
-                     K, up_offset)
+                     K, up_offset, rope)
   switch (epi) {
     case EPI_STORE_BF16: SG_LAUNCH(EPI_STORE_BF16); break;
     case EPI_STORE_F32: SG_LAUNCH(EPI_STORE_F32); break;
     case EPI_ADD: SG_LAUNCH(EPI_ADD); break;
     case EPI_SWIGLU: SG_LAUNCH(EPI_SWIGLU); break;
+    case EPI_ROPE: SG_LAUNCH(EPI_ROPE); break;
     default: MIE_FAIL("skinny_gemm: epilogue code %d", epi);
   }
 #undef SG_LAUNCH
@@ -200,9 +243,28 @@ static int launch_epi(int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx
 
 template <int MT>
 static int launch_waves(int waves, int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx, const bf16* W, long ldw,
-                        void* out, long ldo, int M, int N, int K, int up_offset) {
-  if (waves == 8) return launch_epi<MT, 8>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset);
-  return launch_epi<MT, 4>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset);
+                        void* out, long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope) {
+  if (waves == 8) return launch_epi<MT, 8>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
+  return launch_epi<MT, 4>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
+}
+
+static int launch_rows(int tiles, int epi, hipStream_t s, const bf16* X, long ldx, const bf16* W, long ldw, void* out,
+                       long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope) {
+  dim3 grid(tiles);
+  const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  // few tiles: more waves per tile, so that enough loads are in flight to fill the memory system
+  const int waves = tiles < 256 ? 8 : 4;
+  if (MT == 1) return launch_waves<1>(waves, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
+  if (MT == 2) return launch_waves<2>(waves, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
+  return launch_waves<4>(waves, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
+}
+
+static int check_operands(const char* what, const void* X, long ldx, const void* W, long ldw, int M, int K) {
+  if (M > 64) MIE_FAIL("%s: %d rows (at most 64)", what, M);
+  if (K <= 0 || (K & 7)) MIE_FAIL("%s: K = %d must be a positive multiple of 8", what, K);
+  if (ldx < K || ldw < K || (ldw & 7) || (ldx & 7)) MIE_FAIL("%s: leading dims %ld, %ld for K %d", what, ldx, ldw, K);
+  if (((uintptr_t)X | (uintptr_t)W) & 15) MIE_FAIL("%s: operands must be 16-byte aligned", what);
+  return 0;
 }
 
 // X [M, K] and W bfloat16.  epi: 0 bfloat16 y, 1 float32 y, 2 out[m, n] += y (float32), 3 silu(gate) * up with
@@ -210,19 +272,29 @@ static int launch_waves(int waves, int epi, dim3 grid, hipStream_t s, const bf16
 MIE_EXPORT int mie_skinny_gemm(const void* X, long ldx, const void* W, long ldw, void* out, long ldo, int epi, int M,
                                int N, int K, hipStream_t s) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64) MIE_FAIL("skinny_gemm: %d rows (at most 64)", M);
-  if (K <= 0 || (K & 7)) MIE_FAIL("skinny_gemm: K = %d must be a positive multiple of 8", K);
-  if (ldx < K || ldw < K || (ldw & 7) || (ldx & 7)) MIE_FAIL("skinny_gemm: leading dims %ld, %ld for K %d", ldx, ldw, K);
+  if (epi < 0 || epi > EPI_SWIGLU) MIE_FAIL("skinny_gemm: epilogue code %d", epi);
+  if (check_operands("skinny_gemm", X, ldx, W, ldw, M, K)) return -1;
   if (ldo < N) MIE_FAIL("skinny_gemm: output leading dim %ld < %d", ldo, N);
-  if (((uintptr_t)X | (uintptr_t)W) & 15) MIE_FAIL("skinny_gemm: operands must be 16-byte aligned");
-  const int tiles = (N + 15) / 16;
-  dim3 grid(tiles);
-  const bf16* Xb = (const bf16*)X;
-  const bf16* Wb = (const bf16*)W;
-  const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  // few tiles: more waves per tile, so that enough loads are in flight to fill the memory system
-  const int waves = tiles < 256 ? 8 : 4;
-  if (MT == 1) return launch_waves<1>(waves, epi, grid, s, Xb, ldx, Wb, ldw, out, ldo, M, N, K, N);
-  if (MT == 2) return launch_waves<2>(waves, epi, grid, s, Xb, ldx, Wb, ldw, out, ldo, M, N, K, N);
-  return launch_waves<4>(waves, epi, grid, s, Xb, ldx, Wb, ldw, out, ldo, M, N, K, N);
+  RopeArgs none = {};
+  return launch_rows((N + 15) / 16, epi, s, (const bf16*)X, ldx, (const bf16*)W, ldw, out, ldo, M, N, K, N, none);
+}
+
+// The fused q/k/v projection of single-token rows with what follows it: W [(Hq + 2 Hkv) D, K]; rotary
+// (half-split pairs over the whole head, angles from cos/sin [positions, D / 2] float32) on the q and k
+// heads in 32-bit, q [M, Hq D] written to q_out, rotated k and v written to cache slot slots[m]
+// (k_cache [pages, Hkv, page, D], v_cache [pages, Hkv, D, page]).  D must be a multiple of 32.
+MIE_EXPORT int mie_skinny_qkv_rope(const void* X, long ldx, const void* W, long ldw, void* q_out, long ldq,
+                                   const int* positions, const float* cos_t, const float* sin_t, const int* slots,
+                                   void* k_cache, void* v_cache, int M, int Hq, int Hkv, int D, int page, int K,
+                                   hipStream_t s) {
+  if (M <= 0) return 0;
+  if (D <= 0 || (D & 31)) MIE_FAIL("skinny_qkv_rope: head_dim %d must be a multiple of 32", D);
+  if (Hq <= 0 || Hkv <= 0 || page <= 0) MIE_FAIL("skinny_qkv_rope: heads %d / %d, page %d", Hq, Hkv, page);
+  if (!positions || !cos_t || !sin_t || !slots || !k_cache || !v_cache || !q_out) MIE_FAIL("skinny_qkv_rope: null operand");
+  if (check_operands("skinny_qkv_rope", X, ldx, W, ldw, M, K)) return -1;
+  if (ldq < (long)Hq * D) MIE_FAIL("skinny_qkv_rope: q leading dim %ld < %d", ldq, Hq * D);
+  RopeArgs rope = {positions, cos_t, sin_t, slots, (bf16*)k_cache, (bf16*)v_cache, Hq, Hkv, D, page};
+  const int heads = Hq + 2 * Hkv;
+  return launch_rows(heads * (D / 32), EPI_ROPE, s, (const bf16*)X, ldx, (const bf16*)W, ldw, q_out, ldq, M, heads * D, K,
+                     D / 2, rope);
 }

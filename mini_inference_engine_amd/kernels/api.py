@@ -67,6 +67,16 @@ class KernelBackend:
         rotary_dim 0: no rotation.  num_kv_heads 0 (k_cache None): q only, no write."""
         raise NotImplementedError
 
+    def linear_rotary_kv_store(self, x, w_qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
+                               k_cache, v_cache, slot_mapping):
+        """The fused q/k/v projection followed by rotary_kv_store.  Returns a tensor whose first
+        Hq * D columns are the encoded q (the whole qkv, or q alone): a backend may do all of it in
+        one kernel.  ``x`` is a tensor or a Normed."""
+        qkv = self.linear(x, w_qkv)
+        self.rotary_kv_store(qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim, k_cache,
+                             v_cache, slot_mapping)
+        return qkv
+
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
                         window):
         """For token t of row r at position p: softmax over keys max(0, p - window + 1)..p

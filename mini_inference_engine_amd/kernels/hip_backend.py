@@ -89,6 +89,9 @@ class HipBackend(KernelBackend):
             "gemm_bf16": {
                 "mie_skinny_gemm": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_int,
                                     c_void_p],
+                "mie_skinny_qkv_rope": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                        c_void_p],
                 "mie_skinny_max_rows": [],
             },
             "attention_bf16": {
@@ -227,6 +230,38 @@ class HipBackend(KernelBackend):
             out = torch.empty((x.shape[0], intermediate), dtype=torch.bfloat16, device=w_gate_up.device)
             return self._skinny(x, w_gate_up, self.EPI_SWIGLU, out, intermediate)
         return self.silu_mul(self.linear(x, w_gate_up), intermediate)
+
+    def linear_rotary_kv_store(self, x, w_qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
+                               k_cache, v_cache, slot_mapping):
+        Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
+        if isinstance(x, Normed):
+            x = x.materialize()
+        fused = (Hkv > 0 and rotary_dim == D and D % 32 == 0 and self._skinny_ok(x, w_qkv, None)
+                 and k_cache is not None and k_cache.dtype == torch.bfloat16)
+        if not fused:
+            return super().linear_rotary_kv_store(x, w_qkv, positions, cos, sin, rotary_dim, Hq, Hkv, D, k_cache,
+                                                  v_cache, slot_mapping)
+        self._on_device(x, w_qkv, positions, cos, sin, k_cache, v_cache, slot_mapping)
+        M, K = x.shape
+        if tuple(w_qkv.shape) != ((Hq + 2 * Hkv) * D, K):
+            raise ValueError(f"linear_rotary_kv_store: w {tuple(w_qkv.shape)} for {Hq}+2x{Hkv} heads of {D}, K {K}")
+        page = k_cache.shape[2]
+        for name, t, want in (("k_cache", k_cache, (k_cache.shape[0], Hkv, page, D)),
+                              ("v_cache", v_cache, (k_cache.shape[0], Hkv, D, page))):
+            if tuple(t.shape) != want or t.dtype != torch.bfloat16 or not t.is_contiguous():
+                raise ValueError(f"linear_rotary_kv_store: {name} {tuple(t.shape)} {t.dtype}, expected {want}")
+        for name, t in (("cos", cos), ("sin", sin)):
+            if t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != D // 2 or not t.is_contiguous():
+                raise ValueError(f"linear_rotary_kv_store: {name} must be contiguous float32 [positions, {D // 2}]")
+        for name, t in (("positions", positions), ("slot_mapping", slot_mapping)):
+            if t.dtype != torch.int32 or t.shape[0] != M or not t.is_contiguous():
+                raise ValueError(f"linear_rotary_kv_store: {name} must be contiguous int32 [{M}]")
+        q = torch.empty((M, Hq * D), dtype=torch.bfloat16, device=x.device)
+        lib = self.lib("gemm_bf16")
+        library.check(lib, lib.mie_skinny_qkv_rope(
+            _ptr(x), x.stride(0), _ptr(w_qkv), w_qkv.stride(0), _ptr(q), q.stride(0), _ptr(positions), _ptr(cos),
+            _ptr(sin), _ptr(slot_mapping), _ptr(k_cache), _ptr(v_cache), M, Hq, Hkv, D, page, K, self._stream()))
+        return q
 
     def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
                         k_cache, v_cache, slot_mapping):

@@ -56,11 +56,11 @@ class Attention(Mixer):
         ops = self.ops
         if cache.read_only == self.has_kv:
             raise ValueError("an attention part with k/v projections owns its cache; one without reads another's")
-        qkv = ops.linear(x, self.w_qkv)
         group = step.groups[cache.group]
         kv_heads_in_row = self.num_kv_heads if self.has_kv else 0
         k_cache, v_cache, slots = (cache.k, cache.v, group.slot_mapping) if self.has_kv else (None, None, None)
-        self.position.encode_and_store(ops, qkv, step, self.num_heads, kv_heads_in_row, k_cache, v_cache, slots)
+        qkv = self.position.project_encode_store(ops, x, self.w_qkv, step, self.num_heads, kv_heads_in_row,
+                                                 k_cache, v_cache, slots)
         out = ops.paged_attention(qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v,
                                   group, step, self.scale, self.window)
         return ops.linear(out, self.w_o, add_to=add_to)

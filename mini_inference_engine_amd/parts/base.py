@@ -15,9 +15,11 @@ Norm.forward(x, residual, rows=None) -> y
     produced and the stream is left untouched.  Norm.lazy(...) returns the same
     as a kernels.api.Normed, for parts that set ``lazy_input`` and hand it to
     their first ``ops.linear`` (norm and product then run as one kernel).
-PositionEncoding.encode_and_store(ops, qkv, step, layout, cache, slots)
+PositionEncoding.encode_and_store(ops, qkv, step, n_q_heads, n_kv_heads, k_cache, v_cache, slots)
     Encodes q and k inside the fused projection output in place, as a function of
     each token's absolute position only, and writes k, v to the cache.
+    project_encode_store(ops, x, w_qkv, ...) does the projection too (default: linear,
+    then encode_and_store) and returns a tensor whose first Hq * D columns are q.
 Mixer.forward(x, step, cache, add_to=None) -> y or None     [T, width] -> [T, width]
     Must accept a portion that starts anywhere in a request and leave its cache
     or state as if the request had been fed whole.  ``add_to`` is the stream the
@@ -134,7 +136,14 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    pass
+    def encode_and_store(self, ops, qkv, step, num_q_heads, num_kv_heads, k_cache, v_cache, slots):
+        raise NotImplementedError
+
+    def project_encode_store(self, ops, x, w_qkv, step, num_q_heads, num_kv_heads, k_cache, v_cache, slots):
+        """Default: the projection, then encode_and_store on its output."""
+        qkv = ops.linear(x, w_qkv)
+        self.encode_and_store(ops, qkv, step, num_q_heads, num_kv_heads, k_cache, v_cache, slots)
+        return qkv
 
 
 class Mixer(Part):

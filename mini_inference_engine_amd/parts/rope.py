@@ -46,6 +46,12 @@ class RotaryHalfSplit(PositionEncoding):
         ops.rotary_kv_store(qkv, step.positions, self.cos, self.sin, self.rotary_dim, num_q_heads,
                             num_kv_heads, self.head_dim, k_cache, v_cache, slots)
 
+    def project_encode_store(self, ops, x, w_qkv, step, num_q_heads, num_kv_heads, k_cache, v_cache, slots):
+        """Projection, encoding and cache write together; returns a tensor whose first Hq * D columns
+        are the encoded q.  The backend may run it as one kernel."""
+        return ops.linear_rotary_kv_store(x, w_qkv, step.positions, self.cos, self.sin, self.rotary_dim, num_q_heads,
+                                          num_kv_heads, self.head_dim, k_cache, v_cache, slots)
+
 
 @register_position_encoding("none")
 class NoPosition(PositionEncoding):
@@ -57,3 +63,7 @@ class NoPosition(PositionEncoding):
     def encode_and_store(self, ops, qkv, step, num_q_heads, num_kv_heads, k_cache, v_cache, slots):
         ops.rotary_kv_store(qkv, step.positions, None, None, 0, num_q_heads, num_kv_heads, self.head_dim,
                             k_cache, v_cache, slots)
+
+    def project_encode_store(self, ops, x, w_qkv, step, num_q_heads, num_kv_heads, k_cache, v_cache, slots):
+        return ops.linear_rotary_kv_store(x, w_qkv, step.positions, None, None, 0, num_q_heads, num_kv_heads,
+                                          self.head_dim, k_cache, v_cache, slots)
