@@ -247,26 +247,26 @@ def test_fused_projection_rotary_store(ops, geom, M):
     pos = torch.randint(0, 300, (M,), device=DEV, dtype=torch.int32)
     slots = (torch.randperm((pages - 1) * page, device=DEV)[:M] + page).to(torch.int32)
     kc, vc = make_cache(pages, Hkv, page, D, torch.bfloat16)
-    kc_ref, vc_ref = kc.clone(), vc.clone()
+    kc_ref, vc_ref = kc.float(), vc.float()
     qkv_ref = ref.ref_linear(x, w, None, torch.float32)
     ref.ref_rotary_kv_store(qkv_ref, pos, cos, sin, D, Hq, Hkv, D, kc_ref, vc_ref, slots)
     out = o.linear_rotary_kv_store(x, w, pos, cos, sin, D, Hq, Hkv, D, kc, vc, slots)
     assert tuple(out.shape) == (M, Hq * D), "the fused kernel returns q alone"
     torch.testing.assert_close(out.float(), qkv_ref[:, :Hq * D], atol=2e-2, rtol=1e-2)
-    torch.testing.assert_close(kc.float(), kc_ref.float(), atol=2e-2, rtol=1e-2)
-    torch.testing.assert_close(vc.float(), vc_ref.float(), atol=2e-2, rtol=1e-2)
-    assert torch.equal(kc[0], kc_ref[0]) and torch.equal(vc[0], vc_ref[0]), "untouched pages stay untouched"
+    torch.testing.assert_close(kc.float(), kc_ref, atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(vc.float(), vc_ref, atol=2e-2, rtol=1e-2)
+    assert torch.equal(kc[0].float(), kc_ref[0]) and torch.equal(vc[0].float(), vc_ref[0]), "untouched pages stay untouched"
     # a head size the fused kernel does not take goes through the separate kernels, same result
     if D == 32:
         cos48, sin48 = (t.to(DEV) for t in rotary_tables(10000.0, 48, 300))
         w48 = (torch.randn((Hq + 2 * Hkv) * 48, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
         kc48, vc48 = make_cache(pages, Hkv, page, 48, torch.bfloat16)
-        kr, vr = kc48.clone(), vc48.clone()
+        kr, vr = kc48.float(), vc48.float()
         full = o.linear_rotary_kv_store(x, w48, pos, cos48, sin48, 48, Hq, Hkv, 48, kc48, vc48, slots)
         assert full.shape[1] == (Hq + 2 * Hkv) * 48
         q_ref = ref.ref_linear(x, w48, None, torch.float32)
         ref.ref_rotary_kv_store(q_ref, pos, cos48, sin48, 48, Hq, Hkv, 48, kr, vr, slots)
-        torch.testing.assert_close(kc48.float(), kr.float(), atol=2e-2, rtol=1e-2)
+        torch.testing.assert_close(kc48.float(), kr, atol=2e-2, rtol=1e-2)
 
 
 def test_rotary_q_only(ops):
