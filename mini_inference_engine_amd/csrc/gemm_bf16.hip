@@ -14,8 +14,10 @@
 // Epilogues: STORE (bfloat16 or float32 y), ADD (r[m, n] += y, the residual add of the 32-bit stream),
 //   SWIGLU (W holds gate rows then up rows; the workgroup takes the matching 16 of each and writes
 //   silu(gate) * up).
-// (An RMSNorm prologue on the 32-bit stream was measured here and dropped: every workgroup redoing the
-// conversion of all of x cost more than a separate norm kernel.)
+//   ROPE (the q/k/v projection: rotary on q and k, cache write of k and v).
+// The RMSNorm between two products is folded into them as well, see NormArgs below.  (A norm prologue that
+// converted the 32-bit stream inside every workgroup was measured and dropped: redoing the conversion of
+// all of x per workgroup cost more than a separate norm kernel.)
 #include "common.hpp"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -48,10 +50,28 @@ struct RopeArgs {
   int Hq, Hkv, D, page;
 };
 
-template <int MT, int EPI, int WAVES>
+// The RMSNorm between two of these products, without a kernel of its own (NF).  The product that adds
+// into the stream (ADD) also writes, for the norm that follows it with weight g, x_next[m, n] =
+// bf16(r[m, n] g[n]) and the sum of r[m, n]^2 over its 16 columns (ss_out [tiles, 64]); the product that
+// consumes the normed value takes x_next as its X, sums ss_in over the tiles and scales its results by
+// rstd[m] = 1 / sqrt(sum / width + eps): rstd is a positive scalar per row, so applying it after the
+// product, to values rounded before it, is the same relative rounding as rounding the normed value.
+struct NormArgs {
+  const void* g;             // ADD: weight of the next norm [N]
+  int g_f32;
+  bf16* x_next;              // ADD: [M, ldx_next]
+  long ldx_next;
+  float* ss_out;             // ADD: [tiles of this product, 64]
+  const float* ss_in;        // others: [ss_tiles, 64], indexed by source row
+  int ss_tiles;
+  float inv_width, eps;
+  const int* rows;           // others: optional gather of X's (and ss_in's) rows, int32 [M]
+};
+
+template <int MT, int EPI, int WAVES, bool NF>
 __global__ void __launch_bounds__(WAVES * 64)
 skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict__ W, long ldw, void* __restrict__ outv,
-                   long ldo, int M, int N, int K, int up_offset, RopeArgs rope) {
+                   long ldo, int M, int N, int K, int up_offset, RopeArgs rope, NormArgs nf) {
   constexpr int NT = (EPI == EPI_SWIGLU || EPI == EPI_ROPE) ? 2 : 1;
   // k-steps per group of loads (two groups are in flight per wave)
 #ifndef SG_U_SCALE
@@ -61,6 +81,7 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
   constexpr int SG_WAVES = WAVES;
   constexpr int SG_THREADS = WAVES * 64;
   __shared__ float s_acc[SG_WAVES][MT][256];
+  __shared__ float s_rstd[MT * 16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kb = lane >> 4;
   int n0 = blockIdx.x * 16;
@@ -87,7 +108,24 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + col;
-    xrow[mt] = X + (size_t)(m < M ? m : 0) * ldx;
+    const int src = m < M ? (NF && EPI != EPI_ADD && nf.rows ? nf.rows[m] : m) : 0;
+    xrow[mt] = X + (size_t)src * ldx;
+  }
+  if (NF && EPI != EPI_ADD) {
+    // rstd of every row: 16 lanes a row, each summing every 16th tile's partial, in a fixed order
+#pragma unroll
+    for (int j = 0; j < (MT * 256 + SG_THREADS - 1) / SG_THREADS; ++j) {
+      const int e = threadIdx.x + j * SG_THREADS;
+      const int mm = (e >> 4) < MT * 16 ? (e >> 4) : 0, sub = e & 15;
+      const int src = mm < M ? (nf.rows ? nf.rows[mm] : mm) : 0;
+      float sum = 0.f;
+      for (int t = sub; t < nf.ss_tiles; t += 16) sum += nf.ss_in[(size_t)t * 64 + src];
+      sum += __shfl_xor(sum, 1, 64);
+      sum += __shfl_xor(sum, 2, 64);
+      sum += __shfl_xor(sum, 4, 64);
+      sum += __shfl_xor(sum, 8, 64);
+      if (sub == 0 && e < MT * 256) s_rstd[mm] = 1.0f / sqrtf(sum * nf.inv_width + nf.eps);
+    }
   }
 
   f32x4 acc[NT][MT];
@@ -176,14 +214,36 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int e = threadIdx.x + j * SG_THREADS;
-    if (e >= MT * 256) continue;
     const int m = e >> 4, n = n0 + (e & 15);
-    if (m >= M || n >= N) continue;
+    const bool live = e < MT * 256 && m < M && n < N;
+    if (EPI == EPI_ADD) {
+      const size_t o = (size_t)m * ldo + n;
+      float r = 0.f;
+      if (live) {
+        r = ((float*)outv)[o] + v[0][j];
+        ((float*)outv)[o] = r;
+      }
+      if (NF) {
+        if (live) {
+          const float g = nf.g_f32 ? ((const float*)nf.g)[n] : __bfloat162float(((const bf16*)nf.g)[n]);
+          nf.x_next[(size_t)m * nf.ldx_next + n] = __float2bfloat16(r * g);
+        }
+        float q = r * r;                       // the 16 lanes of a row: sum of squares over this tile's columns
+        q += __shfl_xor(q, 1, 64);
+        q += __shfl_xor(q, 2, 64);
+        q += __shfl_xor(q, 4, 64);
+        q += __shfl_xor(q, 8, 64);
+        if ((e & 15) == 0 && e < MT * 256 && m < M) nf.ss_out[(size_t)blockIdx.x * 64 + m] = q;
+      }
+      continue;
+    }
+    if (!live) continue;
+    const float rstd = NF ? s_rstd[m] : 1.f;
     const size_t o = (size_t)m * ldo + n;
     if (EPI == EPI_ROPE) {
       const int D = rope.D, half = D >> 1;
       const int head = n / D, jd = n - head * D;         // jd < D / 2: the first of the pair
-      const float x1 = v[0][j], x2 = v[NT - 1][j];
+      const float x1 = v[0][j] * rstd, x2 = v[NT - 1][j] * rstd;
       if (head < rope.Hq + rope.Hkv) {
         const int pos = rope.positions[m];
         const float c = rope.cos_t[(size_t)pos * half + jd], sn = rope.sin_t[(size_t)pos * half + jd];
@@ -207,13 +267,11 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
         vc[(size_t)half * rope.page] = __float2bfloat16(x2);
       }
     } else if (EPI == EPI_STORE_BF16) {
-      ((bf16*)outv)[o] = __float2bfloat16(v[0][j]);
+      ((bf16*)outv)[o] = __float2bfloat16(v[0][j] * rstd);
     } else if (EPI == EPI_STORE_F32) {
-      ((float*)outv)[o] = v[0][j];
-    } else if (EPI == EPI_ADD) {
-      ((float*)outv)[o] += v[0][j];
+      ((float*)outv)[o] = v[0][j] * rstd;
     } else {
-      const float g = v[0][j], u = v[NT - 1][j];
+      const float g = v[0][j] * rstd, u = v[NT - 1][j] * rstd;
       ((bf16*)outv)[o] = __float2bfloat16(g / (1.0f + expf(-g)) * u);
     }
   }
@@ -222,12 +280,12 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
 MIE_EXPORT const char* gemm_bf16_last_error() { return g_mie_error; }
 MIE_EXPORT int mie_skinny_max_rows() { return 64; }
 
-template <int MT, int WAVES>
+template <int MT, int WAVES, bool NF>
 static int launch_epi(int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx, const bf16* W, long ldw, void* out,
-                      long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope) {
-#define SG_LAUNCH(E)                                                                                           \
-  hipLaunchKernelGGL((skinny_gemm_kernel<MT, E, WAVES>), grid, dim3(WAVES * 64), 0, s, X, ldx, W, ldw, out, ldo, M, N, \
-                     K, up_offset, rope)
+                      long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope, const NormArgs& nf) {
+#define SG_LAUNCH(E)                                                                                               \
+  hipLaunchKernelGGL((skinny_gemm_kernel<MT, E, WAVES, NF>), grid, dim3(WAVES * 64), 0, s, X, ldx, W, ldw, out, ldo, M, \
+                     N, K, up_offset, rope, nf)
   switch (epi) {
     case EPI_STORE_BF16: SG_LAUNCH(EPI_STORE_BF16); break;
     case EPI_STORE_F32: SG_LAUNCH(EPI_STORE_F32); break;
@@ -242,21 +300,28 @@ static int launch_epi(int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx
 }
 
 template <int MT>
-static int launch_waves(int waves, int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx, const bf16* W, long ldw,
-                        void* out, long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope) {
-  if (waves == 8) return launch_epi<MT, 8>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
-  return launch_epi<MT, 4>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
+static int launch_waves(int waves, bool fused_norm, int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx,
+                        const bf16* W, long ldw, void* out, long ldo, int M, int N, int K, int up_offset,
+                        const RopeArgs& rope, const NormArgs& nf) {
+  if (fused_norm) {
+    if (waves == 8) return launch_epi<MT, 8, true>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, nf);
+    return launch_epi<MT, 4, true>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, nf);
+  }
+  if (waves == 8) return launch_epi<MT, 8, false>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, nf);
+  return launch_epi<MT, 4, false>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, nf);
 }
 
 static int launch_rows(int tiles, int epi, hipStream_t s, const bf16* X, long ldx, const bf16* W, long ldw, void* out,
-                       long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope) {
+                       long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope, const NormArgs* nf) {
   dim3 grid(tiles);
   const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   // few tiles: more waves per tile, so that enough loads are in flight to fill the memory system
   const int waves = tiles < 256 ? 8 : 4;
-  if (MT == 1) return launch_waves<1>(waves, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
-  if (MT == 2) return launch_waves<2>(waves, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
-  return launch_waves<4>(waves, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope);
+  NormArgs none = {};
+  const NormArgs& n = nf ? *nf : none;
+  if (MT == 1) return launch_waves<1>(waves, nf != nullptr, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n);
+  if (MT == 2) return launch_waves<2>(waves, nf != nullptr, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n);
+  return launch_waves<4>(waves, nf != nullptr, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n);
 }
 
 static int check_operands(const char* what, const void* X, long ldx, const void* W, long ldw, int M, int K) {
@@ -267,26 +332,52 @@ static int check_operands(const char* what, const void* X, long ldx, const void*
   return 0;
 }
 
+// The fused norm, both sides.  Producer (epi 2 only): next_g (weight of the norm that follows, bfloat16 or
+// float32), x_next [M, ldx_next] bfloat16 and ss_out [ceil(N / 16), 64] float32 are written beside the add.
+// Consumer (other epilogues): X is a producer's x_next, ss_in its ss_out with ss_tiles tiles, width the
+// norm's width (= K), rows an optional int32 [M] gather of X's rows.  Pass ss_in = next_g = null for none.
+static int fill_norm_args(NormArgs& nf, int epi, const void* next_g, int next_g_f32, void* x_next, long ldx_next,
+                          float* ss_out, const float* ss_in, int ss_tiles, int width, float eps, const int* rows,
+                          int N) {
+  nf = NormArgs{};
+  if (epi == EPI_ADD) {
+    if (!next_g || !x_next || !ss_out || ldx_next < N) MIE_FAIL("skinny_gemm: fused norm output operands");
+    nf.g = next_g; nf.g_f32 = next_g_f32; nf.x_next = (bf16*)x_next; nf.ldx_next = ldx_next; nf.ss_out = ss_out;
+  } else {
+    if (!ss_in || ss_tiles <= 0 || width <= 0) MIE_FAIL("skinny_gemm: fused norm input operands");
+    nf.ss_in = ss_in; nf.ss_tiles = ss_tiles; nf.inv_width = 1.0f / (float)width; nf.eps = eps; nf.rows = rows;
+  }
+  return 0;
+}
+
 // X [M, K] and W bfloat16.  epi: 0 bfloat16 y, 1 float32 y, 2 out[m, n] += y (float32), 3 silu(gate) * up with
 // W = [gate rows (N of them); up rows] and N = the intermediate size.
 MIE_EXPORT int mie_skinny_gemm(const void* X, long ldx, const void* W, long ldw, void* out, long ldo, int epi, int M,
-                               int N, int K, hipStream_t s) {
+                               int N, int K, const void* next_g, int next_g_f32, void* x_next, long ldx_next,
+                               float* ss_out, const float* ss_in, int ss_tiles, float eps, const int* rows,
+                               hipStream_t s) {
   if (M <= 0 || N <= 0) return 0;
   if (epi < 0 || epi > EPI_SWIGLU) MIE_FAIL("skinny_gemm: epilogue code %d", epi);
   if (check_operands("skinny_gemm", X, ldx, W, ldw, M, K)) return -1;
   if (ldo < N) MIE_FAIL("skinny_gemm: output leading dim %ld < %d", ldo, N);
   RopeArgs none = {};
-  return launch_rows((N + 15) / 16, epi, s, (const bf16*)X, ldx, (const bf16*)W, ldw, out, ldo, M, N, K, N, none);
+  NormArgs nf;
+  const bool fused = next_g || ss_in;
+  if (fused && fill_norm_args(nf, epi, next_g, next_g_f32, x_next, ldx_next, ss_out, ss_in, ss_tiles, K, eps, rows, N)) return -1;
+  if (!fused && rows) MIE_FAIL("skinny_gemm: a row gather comes with the fused norm only");
+  return launch_rows((N + 15) / 16, epi, s, (const bf16*)X, ldx, (const bf16*)W, ldw, out, ldo, M, N, K, N, none,
+                     fused ? &nf : nullptr);
 }
 
 // The fused q/k/v projection of single-token rows with what follows it: W [(Hq + 2 Hkv) D, K]; rotary
 // (half-split pairs over the whole head, angles from cos/sin [positions, D / 2] float32) on the q and k
 // heads in 32-bit, q [M, Hq D] written to q_out, rotated k and v written to cache slot slots[m]
 // (k_cache [pages, Hkv, page, D], v_cache [pages, Hkv, D, page]).  D must be a multiple of 32.
+// With ss_in: X is a fused-norm producer's x_next (see above).
 MIE_EXPORT int mie_skinny_qkv_rope(const void* X, long ldx, const void* W, long ldw, void* q_out, long ldq,
                                    const int* positions, const float* cos_t, const float* sin_t, const int* slots,
                                    void* k_cache, void* v_cache, int M, int Hq, int Hkv, int D, int page, int K,
-                                   hipStream_t s) {
+                                   const float* ss_in, int ss_tiles, float eps, hipStream_t s) {
   if (M <= 0) return 0;
   if (D <= 0 || (D & 31)) MIE_FAIL("skinny_qkv_rope: head_dim %d must be a multiple of 32", D);
   if (Hq <= 0 || Hkv <= 0 || page <= 0) MIE_FAIL("skinny_qkv_rope: heads %d / %d, page %d", Hq, Hkv, page);
@@ -295,6 +386,8 @@ MIE_EXPORT int mie_skinny_qkv_rope(const void* X, long ldx, const void* W, long 
   if (ldq < (long)Hq * D) MIE_FAIL("skinny_qkv_rope: q leading dim %ld < %d", ldq, Hq * D);
   RopeArgs rope = {positions, cos_t, sin_t, slots, (bf16*)k_cache, (bf16*)v_cache, Hq, Hkv, D, page};
   const int heads = Hq + 2 * Hkv;
+  NormArgs nf;
+  if (ss_in && fill_norm_args(nf, EPI_ROPE, nullptr, 0, nullptr, 0, nullptr, ss_in, ss_tiles, K, eps, nullptr, heads * D)) return -1;
   return launch_rows(heads * (D / 32), EPI_ROPE, s, (const bf16*)X, ldx, (const bf16*)W, ldw, q_out, ldq, M, heads * D, K,
-                     D / 2, rope);
+                     D / 2, rope, ss_in ? &nf : nullptr);
 }

@@ -8,15 +8,32 @@ Every op runs on the current stream and allocates its outputs with torch.
 """
 from __future__ import annotations
 
+from dataclasses import dataclass
+from typing import Any
+
+
+@dataclass
+class Sink:
+    """Where a part's last product goes: added into the float32 ``stream``; and, if the block knows it,
+    the norm that will read the stream next (its weight and eps), so that a backend can prepare that
+    norm's input in the same kernel."""
+    stream: Any
+    norm_weight: Any = None
+    norm_eps: float = 0.0
+
 
 class Normed:
     """A normalised input that is not computed yet: rmsnorm(residual (+ pending)) * weight, of all
     rows or of ``rows``.  A backend's ``linear`` may take it whole (norm and product in one kernel);
     anything else calls ``materialize()``, which also performs the pending add exactly once."""
 
-    def __init__(self, ops, pending, residual, weight, eps, rows=None):
+    def __init__(self, ops, pending, residual, weight, eps, rows=None, ready=None):
         self.ops, self.pending, self.residual, self.weight, self.eps, self.rows = ops, pending, residual, weight, eps, rows
+        self.ready = ready        # backend-private: what an earlier kernel already prepared of this norm
         self._value = None
+
+    def with_rows(self, rows):
+        return Normed(self.ops, self.pending, self.residual, self.weight, self.eps, rows, self.ready)
 
     @property
     def shape(self):
@@ -49,8 +66,9 @@ class KernelBackend:
 
     def linear(self, x, w, bias=None, out_dtype=None, add_to=None):
         """y = x w^T (+ bias); w [out, in]; 32-bit accumulation.  ``x`` is a tensor or a Normed.
-        With ``add_to`` (the float32 stream [T, out]) the backend may add y into it in place and
-        return None; if it returns a tensor, the caller still has to add it."""
+        With ``add_to`` (the float32 stream [T, out], or a Sink around it) the backend may add y into
+        the stream in place and return None, or, for a Sink that names the next norm, a Normed of the
+        updated stream for that norm; if it returns a plain tensor, the caller still has to add it."""
         raise NotImplementedError
 
     def linear_silu_mul(self, x, w_gate_up, intermediate):

@@ -16,7 +16,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 import torch
 
 from . import library
-from .api import KernelBackend, Normed
+from .api import KernelBackend, Normed, Sink
 
 F32, BF16 = 0, 1
 
@@ -88,10 +88,11 @@ class HipBackend(KernelBackend):
             },
             "gemm_bf16": {
                 "mie_skinny_gemm": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_int,
+                                    c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p,
                                     c_void_p],
                 "mie_skinny_qkv_rope": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                        c_void_p],
+                                        c_void_p, c_int, c_float, c_void_p],
                 "mie_skinny_max_rows": [],
             },
             "attention_bf16": {
@@ -170,39 +171,74 @@ class HipBackend(KernelBackend):
     SKINNY_MAX_ROWS = 16      # above this the library product is faster than the fused kernel as it stands
     EPI_BF16, EPI_F32, EPI_ADD, EPI_SWIGLU = 0, 1, 2, 3
 
-    def _skinny_ok(self, x, w, bias) -> bool:
+    def _skinny_ok(self, x, w, bias, rows=None) -> bool:
         """Whether the fused few-row kernel takes this product (x a bfloat16 tensor)."""
+        m = x.shape[0] if rows is None else rows.shape[0]
         return (not self.true_fp32 and bias is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
-                and x.shape[0] <= self.SKINNY_MAX_ROWS and w.shape[1] % 8 == 0 and w.stride(0) % 8 == 0
+                and m <= self.SKINNY_MAX_ROWS and x.shape[0] <= 64 and w.shape[1] % 8 == 0 and w.stride(0) % 8 == 0
                 and x.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0)
 
-    def _skinny(self, x, w, epi, out, n_out):
+    def _prepared(self, x, w, bias):
+        """If ``x`` is a Normed whose input an earlier product already prepared (weighted, rounded values
+        and per-tile sums of squares) and the fused kernel takes the product: that preparation."""
+        if (isinstance(x, Normed) and x.ready is not None and x.pending is None and x._value is None
+                and self._skinny_ok(x.ready["x"], w, bias, x.rows)):
+            return x.ready
+        return None
+
+    def _skinny(self, x, w, epi, out, n_out, sink=None, prepared=None, rows=None, eps=0.0):
+        """One launch of the few-row kernel.  ``sink`` naming a norm: also prepare that norm's input
+        (returned).  ``prepared``: x is such a preparation; the norm is finished inside this product."""
         lib = self.lib("gemm_bf16")
+        M = x.shape[0] if rows is None else rows.shape[0]
+        made = None
+        norm_args = [None, 0, None, 0, None, None, 0, 0.0, None]
+        if sink is not None and sink.norm_weight is not None:
+            g = sink.norm_weight
+            tiles = -(-n_out // 16)
+            made = {"x": torch.empty((M, n_out), dtype=torch.bfloat16, device=w.device),
+                    "ss": torch.empty((tiles, 64), dtype=torch.float32, device=w.device), "tiles": tiles}
+            norm_args = [_ptr(g), int(g.dtype == torch.float32), _ptr(made["x"]), n_out, _ptr(made["ss"]), None, 0,
+                         0.0, None]
+        elif prepared is not None:
+            norm_args = [None, 0, None, 0, None, _ptr(prepared["ss"]), prepared["tiles"], float(eps), _ptr(rows)]
         library.check(lib, lib.mie_skinny_gemm(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), epi,
-                                               x.shape[0], n_out, w.shape[1], self._stream()))
-        return out
+                                               M, n_out, w.shape[1], *norm_args, self._stream()))
+        return made
 
     def linear(self, x, w, bias=None, out_dtype=None, add_to=None):
-        self._on_device(w, bias, add_to)
+        self._on_device(w, bias)
         _rows_ok(w, "linear: w")
         out_dtype = out_dtype or self.act_dtype
         M, K = x.shape
         if K != w.shape[1]:
             raise ValueError(f"linear: x {tuple(x.shape)} against w {tuple(w.shape)}")
         N = w.shape[0]
-        if add_to is not None and (add_to.dtype != torch.float32 or tuple(add_to.shape) != (M, N)
-                                   or not add_to.is_contiguous()):
-            raise ValueError(f"linear: add_to must be the contiguous float32 stream {(M, N)}")
+        sink = add_to if isinstance(add_to, Sink) or add_to is None else Sink(add_to)
+        if sink is not None:
+            st = sink.stream
+            self._on_device(st)
+            if st.dtype != torch.float32 or tuple(st.shape) != (M, N) or not st.is_contiguous():
+                raise ValueError(f"linear: add_to must be the contiguous float32 stream {(M, N)}")
+        prepared = self._prepared(x, w, bias)
+        if prepared is not None and sink is None and out_dtype in (torch.bfloat16, torch.float32):
+            out = torch.empty((M, N), dtype=out_dtype, device=w.device)
+            self._skinny(prepared["x"], w, self.EPI_BF16 if out_dtype == torch.bfloat16 else self.EPI_F32, out, N,
+                         prepared=prepared, rows=x.rows, eps=x.eps)
+            return out
         if isinstance(x, Normed):
             x = x.materialize()
         self._on_device(x)
         _rows_ok(x, "linear: x")
         if self._skinny_ok(x, w, bias) and out_dtype in (torch.bfloat16, torch.float32):
-            if add_to is not None:
-                self._skinny(x, w, self.EPI_ADD, add_to, N)
-                return None
+            if sink is not None:
+                made = self._skinny(x, w, self.EPI_ADD, sink.stream, N, sink=sink)
+                if made is None:
+                    return None
+                return Normed(self, None, sink.stream, sink.norm_weight, sink.norm_eps, ready=made)
             out = torch.empty((M, N), dtype=out_dtype, device=w.device)
-            return self._skinny(x, w, self.EPI_BF16 if out_dtype == torch.bfloat16 else self.EPI_F32, out, N)
+            self._skinny(x, w, self.EPI_BF16 if out_dtype == torch.bfloat16 else self.EPI_F32, out, N)
+            return out
         if not self.true_fp32 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
             # library matrix product, 32-bit accumulation, as the reference's F.linear
             y = torch.nn.functional.linear(x, w, None if bias is None else bias.to(torch.bfloat16))
@@ -224,20 +260,32 @@ class HipBackend(KernelBackend):
             raise ValueError(f"linear_silu_mul: weight of {w_gate_up.shape[0]} rows for intermediate {intermediate}")
         if x.shape[1] != w_gate_up.shape[1]:
             raise ValueError(f"linear_silu_mul: x {tuple(x.shape)} against w {tuple(w_gate_up.shape)}")
+        prepared = self._prepared(x, w_gate_up, None)
+        if prepared is not None:
+            out = torch.empty((x.shape[0], intermediate), dtype=torch.bfloat16, device=w_gate_up.device)
+            self._skinny(prepared["x"], w_gate_up, self.EPI_SWIGLU, out, intermediate, prepared=prepared, rows=x.rows,
+                         eps=x.eps)
+            return out
         if isinstance(x, Normed):
             x = x.materialize()
         if self._skinny_ok(x, w_gate_up, None):
             out = torch.empty((x.shape[0], intermediate), dtype=torch.bfloat16, device=w_gate_up.device)
-            return self._skinny(x, w_gate_up, self.EPI_SWIGLU, out, intermediate)
+            self._skinny(x, w_gate_up, self.EPI_SWIGLU, out, intermediate)
+            return out
         return self.silu_mul(self.linear(x, w_gate_up), intermediate)
 
     def linear_rotary_kv_store(self, x, w_qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
                                k_cache, v_cache, slot_mapping):
         Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
-        if isinstance(x, Normed):
+        can_rope = (Hkv > 0 and rotary_dim == D and D % 32 == 0 and k_cache is not None
+                    and k_cache.dtype == torch.bfloat16)
+        prepared = self._prepared(x, w_qkv, None) if can_rope and getattr(x, "rows", None) is None else None
+        eps = x.eps if prepared is not None else 0.0
+        if prepared is not None:
+            x = prepared["x"]
+        elif isinstance(x, Normed):
             x = x.materialize()
-        fused = (Hkv > 0 and rotary_dim == D and D % 32 == 0 and self._skinny_ok(x, w_qkv, None)
-                 and k_cache is not None and k_cache.dtype == torch.bfloat16)
+        fused = can_rope and self._skinny_ok(x, w_qkv, None)
         if not fused:
             return super().linear_rotary_kv_store(x, w_qkv, positions, cos, sin, rotary_dim, Hq, Hkv, D, k_cache,
                                                   v_cache, slot_mapping)
@@ -260,7 +308,9 @@ class HipBackend(KernelBackend):
         lib = self.lib("gemm_bf16")
         library.check(lib, lib.mie_skinny_qkv_rope(
             _ptr(x), x.stride(0), _ptr(w_qkv), w_qkv.stride(0), _ptr(q), q.stride(0), _ptr(positions), _ptr(cos),
-            _ptr(sin), _ptr(slot_mapping), _ptr(k_cache), _ptr(v_cache), M, Hq, Hkv, D, page, K, self._stream()))
+            _ptr(sin), _ptr(slot_mapping), _ptr(k_cache), _ptr(v_cache), M, Hq, Hkv, D, page, K,
+            _ptr(prepared["ss"]) if prepared else None, prepared["tiles"] if prepared else 0, float(eps),
+            self._stream()))
         return q
 
     def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,

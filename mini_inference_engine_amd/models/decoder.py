@@ -105,8 +105,10 @@ class Decoder:
         spec = self.spec
         residual = spec.embedding.forward(step.input_ids)
         h = None
-        for call, binding in zip(spec.schedule, self.bindings):
-            h, residual = spec.layers[call.layer].forward(h, residual, step, binding)
+        last = len(spec.schedule) - 1
+        for e, (call, binding) in enumerate(zip(spec.schedule, self.bindings)):
+            after = spec.final_norm if e == last else spec.layers[spec.schedule[e + 1].layer].first_norm
+            h, residual = spec.layers[call.layer].forward(h, residual, step, binding, next_norm=after)
         if step.num_logits == 0:
             return None
         return spec.head.forward(spec.final_norm.lazy(h, residual, rows=step.logit_rows))

@@ -22,11 +22,11 @@ PositionEncoding.encode_and_store(ops, qkv, step, n_q_heads, n_kv_heads, k_cache
     then encode_and_store) and returns a tensor whose first Hq * D columns are q.
 Mixer.forward(x, step, cache, add_to=None) -> y or None     [T, width] -> [T, width]
     Must accept a portion that starts anywhere in a request and leave its cache
-    or state as if the request had been fed whole.  ``add_to`` is the stream the
-    block will add y to: a part may pass it to its last ``ops.linear`` and return
-    what that returns (None = already added), or ignore it and return y.
+    or state as if the request had been fed whole.  ``add_to`` (a kernels.api.Sink)
+    is where the block will add y: a part may pass it to its last ``ops.linear`` and
+    return what that returns (None or a Normed = already added), or ignore it and return y.
 FeedForward.forward(x, step, add_to=None) -> y or None       token-wise
-Block.forward(h, residual, step, cache) -> (h, residual)
+Block.forward(h, residual, step, cache, next_norm=None) -> (h, residual)
 """
 from __future__ import annotations
 
@@ -165,8 +165,9 @@ class FeedForward(Part):
 
 class Block(Part):
     mixer: Mixer
+    first_norm = None       # the norm a block applies to the stream first, if it wants the block before it to know
 
-    def forward(self, h, residual, step, cache: CacheBinding):
+    def forward(self, h, residual, step, cache: CacheBinding, next_norm=None):
         raise NotImplementedError
 
 

@@ -22,8 +22,16 @@ class RMSNorm(Norm):
     def params(self):
         return [ParamSpec.single("weight", self.weight_name, (self.width,))]
 
-    def forward(self, x, residual, rows=None, out_dtype=None):
-        return self.ops.add_rmsnorm(x, residual, self.weight, self.eps, out_dtype=out_dtype, rows=rows)
-
     def lazy(self, x, residual, rows=None):
+        if isinstance(x, Normed):
+            # the product before this norm already added its result to the stream (and may have prepared
+            # this very norm's input)
+            if x.weight is self.weight and x.residual is residual and x.eps == self.eps and x.pending is None:
+                return x if rows is None else x.with_rows(rows)
+            x = None
         return Normed(self.ops, x, residual, self.weight, self.eps, rows)
+
+    def forward(self, x, residual, rows=None, out_dtype=None):
+        if isinstance(x, Normed):
+            return self.lazy(x, residual, rows).materialize(out_dtype)
+        return self.ops.add_rmsnorm(x, residual, self.weight, self.eps, out_dtype=out_dtype, rows=rows)

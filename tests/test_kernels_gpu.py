@@ -191,6 +191,64 @@ def test_lazy_norm_input_adds_once(ops):
     torch.testing.assert_close(lazy.residual, stream + pending.float())
 
 
+@pytest.mark.parametrize("g_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M, width, inner", [(1, 64, 176), (8, 2048, 512), (16, 96, 64), (40, 120, 331), (64, 200, 48)])
+def test_norm_folded_into_neighbouring_products(ops, M, width, inner, g_dtype):
+    """stream += x W1^T, then the RMSNorm of the stream, then a product: the norm has no kernel of its own.
+    The first product prepares its input (values times weight, rounded; sums of squares per tile), the
+    second applies 1 / sqrt(mean + eps) to its sums."""
+    from mini_inference_engine_amd.kernels.api import Sink
+    o = ops[torch.bfloat16]
+    torch.manual_seed(M + width)
+    x = torch.randn(M, inner, device=DEV).to(torch.bfloat16)
+    w1 = (torch.randn(width, inner, device=DEV) / math.sqrt(inner)).to(torch.bfloat16)
+    g = (1 + 0.1 * torch.randn(width, device=DEV)).to(g_dtype)
+    stream = torch.randn(M, width, device=DEV)
+    expect_stream = stream.double() + x.double() @ w1.double().T
+    normed_in = o.linear(x, w1, add_to=Sink(stream, g, 1e-5))
+    assert normed_in is not None and normed_in.ready is not None, "the fused kernel must have prepared the norm"
+    torch.testing.assert_close(stream.double(), expect_stream, atol=2e-3, rtol=2e-3)
+    xn = ref.ref_add_rmsnorm(None, stream.clone(), g, 1e-5, torch.float64)
+    # consumer 1: plain product, float32 out, gathered rows (the head on wanted rows)
+    w2 = (torch.randn(77, width, device=DEV) / math.sqrt(width)).to(torch.bfloat16)
+    rows = torch.tensor([M - 1, 0, M // 2], device=DEV, dtype=torch.int32)
+    y = o.linear(normed_in.with_rows(rows), w2, out_dtype=torch.float32)
+    torch.testing.assert_close(y.double(), xn[rows.long()] @ w2.double().T, atol=2e-2, rtol=1e-2)
+    # consumer 2: gate/up with SwiGLU
+    w3 = (torch.randn(2 * 48, width, device=DEV) / math.sqrt(width)).to(torch.bfloat16)
+    a = o.linear_silu_mul(normed_in, w3, 48)
+    gu = xn @ w3.double().T
+    torch.testing.assert_close(a.double(), torch.nn.functional.silu(gu[:, :48]) * gu[:, 48:], atol=3e-2, rtol=2e-2)
+    # the same Normed, materialised the ordinary way, agrees
+    torch.testing.assert_close(normed_in.materialize().double(), xn, atol=2e-2, rtol=1e-2)
+
+
+def test_norm_folded_into_projection_rotary_store(ops):
+    from mini_inference_engine_amd.kernels.api import Sink
+    from mini_inference_engine_amd.parts.rope import rotary_tables
+    o = ops[torch.bfloat16]
+    torch.manual_seed(3)
+    M, width, Hq, Hkv, D, page, pages = 8, 256, 4, 2, 64, 16, 6
+    cos, sin = (t.to(DEV) for t in rotary_tables(10000.0, D, 300))
+    x = torch.randn(M, 96, device=DEV).to(torch.bfloat16)
+    w1 = (torch.randn(width, 96, device=DEV) / 10).to(torch.bfloat16)
+    g = (1 + 0.1 * torch.randn(width, device=DEV)).to(torch.bfloat16)
+    stream = torch.randn(M, width, device=DEV)
+    normed_in = o.linear(x, w1, add_to=Sink(stream, g, 1e-6))
+    w = (torch.randn((Hq + 2 * Hkv) * D, width, device=DEV) / 16).to(torch.bfloat16)
+    pos = torch.randint(0, 300, (M,), device=DEV, dtype=torch.int32)
+    slots = (torch.randperm((pages - 1) * page, device=DEV)[:M] + page).to(torch.int32)
+    kc, vc = make_cache(pages, Hkv, page, D, torch.bfloat16)
+    kc_ref, vc_ref = kc.float(), vc.float()
+    xn = ref.ref_add_rmsnorm(None, stream.clone(), g, 1e-6, torch.float32)
+    qkv_ref = (xn.double() @ w.double().T).float()
+    ref.ref_rotary_kv_store(qkv_ref, pos, cos, sin, D, Hq, Hkv, D, kc_ref, vc_ref, slots)
+    q = o.linear_rotary_kv_store(normed_in, w, pos, cos, sin, D, Hq, Hkv, D, kc, vc, slots)
+    torch.testing.assert_close(q.float(), qkv_ref[:, :Hq * D], atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(kc.float(), kc_ref, atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(vc.float(), vc_ref, atol=2e-2, rtol=1e-2)
+
+
 @pytest.mark.parametrize("M, K, inter", [(1, 64, 176), (8, 2048, 5632), (20, 96, 256), (50, 120, 200), (64, 64, 48)])
 def test_skinny_swiglu(ops, M, K, inter):
     o = ops[torch.bfloat16]

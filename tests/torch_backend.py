@@ -12,7 +12,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from mini_inference_engine_amd.kernels.api import KernelBackend, Normed
+from mini_inference_engine_amd.kernels.api import KernelBackend, Normed, Sink
 
 
 def ref_embedding(ids, table):
@@ -144,8 +144,11 @@ class TorchBackend(KernelBackend):
         if isinstance(x, Normed):
             x = x.materialize()
         y = ref_linear(x, w, bias, out_dtype or self.act_dtype)
-        if add_to is not None and self.adds_in_place:
-            add_to.add_(y.float())
+        sink = add_to if isinstance(add_to, Sink) else (Sink(add_to) if add_to is not None else None)
+        if sink is not None and self.adds_in_place:
+            sink.stream.add_(y.float())
+            if sink.norm_weight is not None:      # as a fusing backend would: the next norm, prepared
+                return Normed(self, None, sink.stream, sink.norm_weight, sink.norm_eps)
             return None
         return y
 
