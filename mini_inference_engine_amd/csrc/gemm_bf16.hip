@@ -111,20 +111,23 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
     const int src = m < M ? (NF && EPI != EPI_ADD && nf.rows ? nf.rows[m] : m) : 0;
     xrow[mt] = X + (size_t)src * ldx;
   }
+  // Fused norm, consuming side: the partial sums of squares are asked for here and used after the main
+  // loop, so that their latency hides behind the weights'.  16 lanes a row, lane sub takes tiles sub,
+  // sub + 16, ...: the first SSP of them now, the rest (widths above 4096) after the loop.
+  constexpr int PER = (MT * 256 + SG_THREADS - 1) / SG_THREADS;
+  constexpr int SSP = 4;
+  float ssp[PER][SSP];
   if (NF && EPI != EPI_ADD) {
-    // rstd of every row: 16 lanes a row, each summing every 16th tile's partial, in a fixed order
 #pragma unroll
-    for (int j = 0; j < (MT * 256 + SG_THREADS - 1) / SG_THREADS; ++j) {
+    for (int j = 0; j < PER; ++j) {
       const int e = threadIdx.x + j * SG_THREADS;
       const int mm = (e >> 4) < MT * 16 ? (e >> 4) : 0, sub = e & 15;
       const int src = mm < M ? (nf.rows ? nf.rows[mm] : mm) : 0;
-      float sum = 0.f;
-      for (int t = sub; t < nf.ss_tiles; t += 16) sum += nf.ss_in[(size_t)t * 64 + src];
-      sum += __shfl_xor(sum, 1, 64);
-      sum += __shfl_xor(sum, 2, 64);
-      sum += __shfl_xor(sum, 4, 64);
-      sum += __shfl_xor(sum, 8, 64);
-      if (sub == 0 && e < MT * 256) s_rstd[mm] = 1.0f / sqrtf(sum * nf.inv_width + nf.eps);
+#pragma unroll
+      for (int i = 0; i < SSP; ++i) {
+        const int t = sub + 16 * i;
+        ssp[j][i] = nf.ss_in[(size_t)(t < nf.ss_tiles ? t : 0) * 64 + src];
+      }
     }
   }
 
@@ -186,8 +189,28 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
     multiply(g1);
   }
 
+  if (NF && EPI != EPI_ADD) {
+    // 1 / sqrt(mean of squares + eps) of every row, summed in a fixed order
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = threadIdx.x + j * SG_THREADS;
+      const int mm = (e >> 4) < MT * 16 ? (e >> 4) : 0, sub = e & 15;
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < SSP; ++i) sum += sub + 16 * i < nf.ss_tiles ? ssp[j][i] : 0.f;
+      if (nf.ss_tiles > 16 * SSP) {
+        const int src = mm < M ? (nf.rows ? nf.rows[mm] : mm) : 0;
+        for (int t = sub + 16 * SSP; t < nf.ss_tiles; t += 16) sum += nf.ss_in[(size_t)t * 64 + src];
+      }
+      sum += __shfl_xor(sum, 1, 64);
+      sum += __shfl_xor(sum, 2, 64);
+      sum += __shfl_xor(sum, 4, 64);
+      sum += __shfl_xor(sum, 8, 64);
+      if (sub == 0 && e < MT * 256) s_rstd[mm] = 1.0f / sqrtf(sum * nf.inv_width + nf.eps);
+    }
+  }
+
   // sum the waves, tile after tile, each thread owning elements (m, n) = (e / 16, e % 16)
-  constexpr int PER = (MT * 256 + SG_THREADS - 1) / SG_THREADS;
   float v[NT][PER];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {

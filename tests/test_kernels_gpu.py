@@ -192,7 +192,7 @@ def test_lazy_norm_input_adds_once(ops):
 
 
 @pytest.mark.parametrize("g_dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("M, width, inner", [(1, 64, 176), (8, 2048, 512), (16, 96, 64), (40, 120, 331), (64, 200, 48)])
+@pytest.mark.parametrize("M, width, inner", [(1, 64, 176), (8, 2048, 512), (16, 96, 64), (5, 120, 328), (13, 200, 48), (3, 4160, 64)])
 def test_norm_folded_into_neighbouring_products(ops, M, width, inner, g_dtype):
     """stream += x W1^T, then the RMSNorm of the stream, then a product: the norm has no kernel of its own.
     The first product prepares its input (values times weight, rounded; sums of squares per tile), the
@@ -598,6 +598,30 @@ def test_sample_greedy_and_ties(ops):
     expect = logits.argmax(-1)
     expect[3], expect[4] = 100, 0
     assert out.tolist() == expect.tolist()
+
+
+@pytest.mark.parametrize("V, ld", [(4099, 4100), (8192, 8192), (4097, 4097), (5, 8)])
+def test_sample_wide_rows(ops, V, ld):
+    """Rows read four values at a time and one at a time, with a tail: the winner may sit anywhere."""
+    torch.manual_seed(V)
+    full = torch.randn(6, ld, device=DEV)
+    full[:, V:] = 100.0                                  # beyond the vocabulary: never looked at
+    logits = full[:, :V]
+    places = [0, V - 1, max(V - 2, 0), V // 2, min(V & ~3, V - 1), min(V - 1, 4095)]
+    for r, v in enumerate(places):
+        logits[r, v] = 30.0
+    zeros = torch.zeros(6, device=DEV)
+    out = ops[torch.float32].sample(logits, zeros, torch.zeros(6, dtype=torch.int64, device=DEV),
+                                    torch.zeros(6, dtype=torch.int32, device=DEV))
+    assert out.tolist() == places
+    temps = torch.full((6,), 0.9, device=DEV)
+    seeds = torch.arange(6, dtype=torch.int64, device=DEV) + 11
+    ctrs = torch.arange(6, dtype=torch.int32, device=DEV)
+    noisy = (torch.randn(6, ld, device=DEV) * 2)[:, :V]
+    out = ops[torch.float32].sample(noisy, temps, seeds, ctrs).tolist()
+    for r in range(6):
+        z = ref.ref_perturbed(noisy[r], 0.9, int(seeds[r]), int(ctrs[r]))
+        assert float(z.max() - z[out[r]]) <= 1e-4, f"row {r}: chose {out[r]}, best {int(z.argmax())}"
 
 
 def test_sample_noise_matches_specification(ops):
