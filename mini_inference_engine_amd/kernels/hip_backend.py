@@ -197,7 +197,7 @@ class HipBackend(KernelBackend):
             g = sink.norm_weight
             tiles = -(-n_out // 16)
             made = {"x": torch.empty((M, n_out), dtype=torch.bfloat16, device=w.device),
-                    "ss": torch.empty((tiles, 64), dtype=torch.float32, device=w.device), "tiles": tiles}
+                    "ss": torch.empty((M, (tiles + 3) // 4 * 4), dtype=torch.float32, device=w.device), "tiles": tiles}
             norm_args = [_ptr(g), int(g.dtype == torch.float32), _ptr(made["x"]), n_out, _ptr(made["ss"]), None, 0,
                          0.0, None]
         elif prepared is not None:
@@ -277,7 +277,7 @@ class HipBackend(KernelBackend):
     def linear_rotary_kv_store(self, x, w_qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
                                k_cache, v_cache, slot_mapping):
         Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
-        can_rope = (Hkv > 0 and rotary_dim == D and D % 32 == 0 and k_cache is not None
+        can_rope = (Hkv > 0 and rotary_dim == D and D % 16 == 0 and k_cache is not None
                     and k_cache.dtype == torch.bfloat16)
         prepared = self._prepared(x, w_qkv, None) if can_rope and getattr(x, "rows", None) is None else None
         eps = x.eps if prepared is not None else 0.0
