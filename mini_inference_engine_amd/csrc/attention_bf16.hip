@@ -38,13 +38,17 @@ union Frag {
   uint32_t w[4];
 };
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+// two floats to two bfloat16 (round to nearest even, one v_cvt_pk_bf16_f32), low half = a
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-  // round to nearest even, low half = a
-  uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
-  ua += 0x7FFFu + ((ua >> 16) & 1u);
-  ub += 0x7FFFu + ((ub >> 16) & 1u);
-  return (ua >> 16) | (ub & 0xFFFF0000u);
+  const float2_t f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
 }
+
+// 2^x by the hardware instruction alone: results below 2^-126 are flushed to 0, which a softmax weight may be
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __global__ void __launch_bounds__(NW * 64)
 decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* __restrict__ k_cache,
@@ -275,7 +279,10 @@ merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ 
 // O^T[d, query] += V^T . P^T, so softmax state is again one value per lane (its query).  A wave owns
 // PF_NT tiles of 16 queries x 1 head (heads of one kv group and/or consecutive query tiles) and
 // walks the keys its queries can see in blocks of 32; each key and value fragment it loads feeds all
-// its tiles.  No LDS, no barriers: waves are independent.
+// its tiles, and the fragments of the next block are requested before the current one is computed.
+// No LDS, no barriers: waves are independent.  Workgroups are numbered from the last queries of a row
+// (most keys) to the first, so the long ones start first.  A block every query of a tile sees whole
+// takes a path without masks.  The running maximum m is kept in units of scale * log2(e).
 constexpr int PF_NT = D <= 64 ? 4 : (D <= 128 ? 2 : 1);
 
 __global__ void __launch_bounds__(256)
@@ -291,12 +298,12 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
   const int col = lane & 15, kb = lane >> 4;
   const int t0 = row_start[row], q_len = row_start[row + 1] - t0, p0 = row_position[row];
   const int qpw = PF_NT / hpw;                              // query tiles per wave
-  const int qt0 = (blockIdx.x * 4 + wave) * qpw;            // first query tile of this wave
+  const int qt0 = ((gridDim.x - 1 - blockIdx.x) * 4 + wave) * qpw;   // first query tile of this wave
   if (qt0 * 16 >= q_len) return;
   const int* bt = block_tables + (size_t)row * max_blocks;
 
   bool tile_ok[PF_NT];
-  int qpos[PF_NT], qtok[PF_NT], tile_last[PF_NT], head[PF_NT];
+  int qpos[PF_NT], qtok[PF_NT], tile_first[PF_NT], tile_last[PF_NT], head[PF_NT];
   bool q_ok[PF_NT];
   Frag qf[PF_NT][KS];
 #pragma unroll
@@ -311,6 +318,7 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
     qtok[j] = t0 + qi;
     qpos[j] = p0 + qi;
     const int last_q = (qt * 16 + 15 < q_len ? qt * 16 + 15 : q_len - 1);
+    tile_first[j] = p0 + qt * 16;
     tile_last[j] = p0 + (last_q > 0 ? last_q : 0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -339,99 +347,174 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
     for (int dt = 0; dt < DT; ++dt) O[j][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int blk = kmin & ~(BLOCK_KEYS - 1); blk <= kmax; blk += BLOCK_KEYS) {
-    Frag a[2][KS];
+  // The fragments of one block of 32 keys: requests only (every address is clamped into the row's own
+  // pages, so a block beyond the last key may be asked for and is never used).  The pages of a block
+  // are looked up one block earlier than its fragments are requested.
+  struct KeyBlock {
+    Frag a[2][KS];      // keys: 16 keys x 32 dims each
+    Frag va[DT];        // values: 16 dims x 32 keys each, keys in the order the probabilities sit in registers
+  };
+  struct Pages {
+    int k[2], v[2];     // page of this lane's key in each 16-key tile; page of its two groups of 4 values
+  };
+  auto lookup_pages = [&](Pages& P, int blk) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       int key = blk + 16 * t + col;
       key = key < kmax ? key : kmax;
-      const int pg = bt[key / page];
-      const bf16* kp = k_cache + (((size_t)pg * Hkv + kvh) * page + key % page) * D;
+      P.k[t] = bt[key / page];
+    }
+    const int last = kmax & ~3;
+    int k0 = blk + 4 * kb, k1 = blk + 16 + 4 * kb;
+    k0 = k0 < last ? k0 : last;
+    k1 = k1 < last ? k1 : last;
+    P.v[0] = bt[k0 / page];
+    P.v[1] = bt[k1 / page];
+  };
+  auto load_block = [&](KeyBlock& B, const Pages& P, int blk) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      int key = blk + 16 * t + col;
+      key = key < kmax ? key : kmax;
+      const bf16* kp = k_cache + (((size_t)P.k[t] * Hkv + kvh) * page + key % page) * D;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const int d0 = ks * 32 + kb * 8;
-        a[t][ks].q = make_uint4(0, 0, 0, 0);
-        if (d0 < D) a[t][ks].q = *reinterpret_cast<const uint4*>(kp + d0);
+        B.a[t][ks].q = *reinterpret_cast<const uint4*>(kp + (d0 < D ? d0 : 0));
       }
     }
-    Frag va[DT];
-    {
-      int k0 = blk + 4 * kb, k1 = blk + 16 + 4 * kb;
-      const int last = kmax & ~3;
-      k0 = k0 < last ? k0 : last;
-      k1 = k1 < last ? k1 : last;
-      const int pg0 = bt[k0 / page], pg1 = bt[k1 / page];
-      const bf16* v0 = v_cache + ((size_t)pg0 * Hkv + kvh) * D * page + k0 % page;
-      const bf16* v1 = v_cache + ((size_t)pg1 * Hkv + kvh) * D * page + k1 % page;
+    int k0 = blk + 4 * kb, k1 = blk + 16 + 4 * kb;
+    const int last = kmax & ~3;
+    k0 = k0 < last ? k0 : last;
+    k1 = k1 < last ? k1 : last;
+    const bf16* v0 = v_cache + ((size_t)P.v[0] * Hkv + kvh) * D * page + k0 % page;
+    const bf16* v1 = v_cache + ((size_t)P.v[1] * Hkv + kvh) * D * page + k1 % page;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const size_t drow = (size_t)(dt * 16 + col) * page;
-        va[dt].h[0] = *reinterpret_cast<const uint2*>(v0 + drow);
-        va[dt].h[1] = *reinterpret_cast<const uint2*>(v1 + drow);
-      }
-      if (blk + BLOCK_KEYS > kmax + 1) {
-        // slots after the wave's last key may be stale: zero them (0 * NaN must not reach the sum)
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int jj = 0; jj < 4; ++jj) {
-            const int ka = blk + (jj < 2 ? 0 : 16) + 4 * kb + 2 * (jj & 1);
-            uint32_t w = va[dt].w[jj];
-            if (ka > kmax) w &= 0xFFFF0000u;
-            if (ka + 1 > kmax) w &= 0x0000FFFFu;
-            va[dt].w[jj] = w;
-          }
-      }
+    for (int dt = 0; dt < DT; ++dt) {
+      const size_t drow = (size_t)(dt * 16 + col) * page;
+      B.va[dt].h[0] = *reinterpret_cast<const uint2*>(v0 + drow);
+      B.va[dt].h[1] = *reinterpret_cast<const uint2*>(v1 + drow);
     }
-#pragma unroll
-    for (int j = 0; j < PF_NT; ++j) {
-      if (!tile_ok[j] || blk > tile_last[j]) continue;       // uniform over the wave
-      f32x4 S[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        S[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-          S[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][ks].v, qf[j][ks].v, S[t], 0, 0, 0);
-      }
-      const int hi = qpos[j];
-      const int lo = window > 0 ? hi - window + 1 : 0;
-      float sv[8];
-      bool ok[8];
-      float mx = -INFINITY;
+  };
+
+  // One block for all tiles of the wave, stage by stage (scores of every tile, softmax of every tile,
+  // outputs of every tile), so that the matrix and the vector unit have independent work side by side.
+  auto compute = [&](KeyBlock& B, int blk) {
+    if (D % 32 != 0) {
+      // the last 32-dim step of the keys is half empty: its upper lanes were loaded from dim 0
 #pragma unroll
       for (int t = 0; t < 2; ++t)
+        if ((KS - 1) * 32 + kb * 8 >= D) B.a[t][KS - 1].q = make_uint4(0, 0, 0, 0);
+    }
+    if (blk + BLOCK_KEYS > kmax + 1) {
+      // slots after the wave's last key may be stale: zero them (0 * NaN must not reach the sum)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = blk + 16 * t + 4 * kb + i;
-          ok[t * 4 + i] = key >= lo && key <= hi;
-          sv[t * 4 + i] = ok[t * 4 + i] ? S[t][i] * scale_log2 : -INFINITY;
-          mx = fmaxf(mx, sv[t * 4 + i]);
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const int ka = blk + (jj < 2 ? 0 : 16) + 4 * kb + 2 * (jj & 1);
+          uint32_t w = B.va[dt].w[jj];
+          if (ka > kmax) w &= 0xFFFF0000u;
+          if (ka + 1 > kmax) w &= 0x0000FFFFu;
+          B.va[dt].w[jj] = w;
         }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[j], mx);
-      // a query may see none of this block's keys (it lies before the block, or the block before its window)
-      const float alpha = m_new == -INFINITY ? 1.f : exp2f(m[j] - m_new);
-      float p[8], rs = 0.f;
+    }
+    f32x4 S[PF_NT][2];
+    bool whole = true;      // every query of every tile sees every key of the block (uniform over the wave)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        p[e] = ok[e] ? exp2f(sv[e] - m_new) : 0.f;
-        rs += p[e];
+    for (int j = 0; j < PF_NT; ++j) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        S[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          S[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(B.a[t][ks].v, qf[j][ks].v, S[j][t], 0, 0, 0);
       }
-      rs += __shfl_xor(rs, 16, 64);
-      rs += __shfl_xor(rs, 32, 64);
-      l[j] = l[j] * alpha + rs;
-      m[j] = m_new;
-      Frag pb;
+      whole = whole && (!tile_ok[j] || (blk + BLOCK_KEYS - 1 <= tile_first[j] &&
+                                        (window <= 0 || blk >= tile_last[j] - window + 1)));
+    }
+    float p[PF_NT][8], alpha[PF_NT];
+    if (whole) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) pb.w[e] = pack_bf16(p[2 * e], p[2 * e + 1]);
+      for (int j = 0; j < PF_NT; ++j) {
+        float mx = fmaxf(fmaxf(fmaxf(S[j][0][0], S[j][0][1]), fmaxf(S[j][0][2], S[j][0][3])),
+                         fmaxf(fmaxf(S[j][1][0], S[j][1][1]), fmaxf(S[j][1][2], S[j][1][3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m[j], mx * scale_log2);
+        alpha[j] = fast_exp2(m[j] - m_new);
+        m[j] = m_new;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        O[j][dt] *= alpha;
-        O[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt].v, pb.v, O[j][dt], 0, 0, 0);
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) p[j][t * 4 + i] = fast_exp2(fmaf(S[j][t][i], scale_log2, -m_new));
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < PF_NT; ++j) {
+        const int hi = tile_ok[j] ? qpos[j] : -1;            // a tile that does not exist sees nothing
+        const int lo = window > 0 ? hi - window + 1 : 0;
+        bool ok[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = blk + 16 * t + 4 * kb + i;
+            ok[t * 4 + i] = key >= lo && key <= hi;
+            mx = fmaxf(mx, ok[t * 4 + i] ? S[j][t][i] : -INFINITY);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m[j], mx * scale_log2);
+        // a query may see none of this block's keys (it lies before the block, or the block before its window)
+        alpha[j] = m_new == -INFINITY ? 1.f : fast_exp2(m[j] - m_new);
+        m[j] = m_new;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            p[j][t * 4 + i] = ok[t * 4 + i] ? fast_exp2(fmaf(S[j][t][i], scale_log2, -m_new)) : 0.f;
       }
     }
+    Frag pb[PF_NT];
+    bool moved = false;
+#pragma unroll
+    for (int j = 0; j < PF_NT; ++j) {
+      float rs = ((p[j][0] + p[j][1]) + (p[j][2] + p[j][3])) + ((p[j][4] + p[j][5]) + (p[j][6] + p[j][7]));
+      rs += __shfl_xor(rs, 16, 64);
+      rs += __shfl_xor(rs, 32, 64);
+      l[j] = l[j] * alpha[j] + rs;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pb[j].w[e] = pack_bf16(p[j][2 * e], p[j][2 * e + 1]);
+      moved = moved || alpha[j] != 1.f;
+    }
+    if (__builtin_amdgcn_ballot_w64(moved) != 0) {          // the maxima rarely move after the first blocks
+#pragma unroll
+      for (int j = 0; j < PF_NT; ++j)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) O[j][dt] *= alpha[j];
+    }
+#pragma unroll
+    for (int j = 0; j < PF_NT; ++j)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        O[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(B.va[dt].v, pb[j].v, O[j][dt], 0, 0, 0);
+  };
+
+  KeyBlock b0, b1;
+  Pages pg;
+  const int blk0 = kmin & ~(BLOCK_KEYS - 1);
+  lookup_pages(pg, blk0);
+  load_block(b0, pg, blk0);
+  lookup_pages(pg, blk0 + BLOCK_KEYS);
+  for (int blk = blk0; blk <= kmax; blk += 2 * BLOCK_KEYS) {
+    load_block(b1, pg, blk + BLOCK_KEYS);             // in flight while block 0 is computed
+    lookup_pages(pg, blk + 2 * BLOCK_KEYS);
+    compute(b0, blk);
+    load_block(b0, pg, blk + 2 * BLOCK_KEYS);
+    lookup_pages(pg, blk + 3 * BLOCK_KEYS);
+    if (blk + BLOCK_KEYS <= kmax) compute(b1, blk + BLOCK_KEYS);
   }
 
 #pragma unroll
