@@ -47,6 +47,26 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
 }
 
+// max of two numbers neither of which is a NaN, as one instruction (fmaxf adds two more to quiet NaNs)
+__device__ __forceinline__ float max_nn(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, INFINITY); }
+
+// max / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (one query's or head's lanes), by the lane
+// swaps of gfx950 instead of a trip through the LDS: v_permlane16_swap exchanges the odd 16-lane rows of
+// its first operand with the even rows of its second, v_permlane32_swap the upper half of the first with
+// the lower half of the second; with both operands equal, the pair holds x[l] and x[l ^ 16] (x[l ^ 32]).
+__device__ __forceinline__ float quad_max(float x) {      // no NaN among the values
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = max_nn(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return max_nn(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float quad_sum(float x) {
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // 2^x by the hardware instruction alone: results below 2^-126 are flushed to 0, which a softmax weight may be
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -355,40 +375,50 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
     Frag va[DT];        // values: 16 dims x 32 keys each, keys in the order the probabilities sit in registers
   };
   struct Pages {
-    int k[2], v[2];     // page of this lane's key in each 16-key tile; page of its two groups of 4 values
+    int k[2], koff[2];  // page of this lane's key in each 16-key tile, and the key's place in that page
+    int v[2], voff[2];  // page of its two groups of 4 values, and the first one's place
   };
+  // The block table is walked, not divided into: [walk_start, walk_start + page) is the page that holds
+  // the block looked up last, and a key at most 31 past a block's start lies at most two pages on.
+  const int blk0 = kmin & ~(BLOCK_KEYS - 1);
+  const int last_blk = kmax & ~(BLOCK_KEYS - 1);
+  int walk_idx = blk0 / page, walk_start = walk_idx * page;
   auto lookup_pages = [&](Pages& P, int blk) {
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      int key = blk + 16 * t + col;
-      key = key < kmax ? key : kmax;
-      P.k[t] = bt[key / page];
+    blk = blk < last_blk ? blk : last_blk;           // a block beyond the last key: the last one again
+    while (blk >= walk_start + page) {
+      walk_start += page;
+      ++walk_idx;
     }
     const int last = kmax & ~3;
-    int k0 = blk + 4 * kb, k1 = blk + 16 + 4 * kb;
-    k0 = k0 < last ? k0 : last;
-    k1 = k1 < last ? k1 : last;
-    P.v[0] = bt[k0 / page];
-    P.v[1] = bt[k1 / page];
+    int keys[4] = {blk + col, blk + 16 + col, blk + 4 * kb, blk + 16 + 4 * kb};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int bound = i < 2 ? kmax : last;
+      const int key = keys[i] < bound ? keys[i] : bound;
+      const int rel = key - walk_start;
+      const int w = (rel >= page ? 1 : 0) + (rel >= 2 * page ? 1 : 0);
+      const int pg = bt[walk_idx + w];
+      if (i < 2) {
+        P.k[i] = pg;
+        P.koff[i] = rel - w * page;
+      } else {
+        P.v[i - 2] = pg;
+        P.voff[i - 2] = rel - w * page;
+      }
+    }
   };
-  auto load_block = [&](KeyBlock& B, const Pages& P, int blk) {
+  auto load_block = [&](KeyBlock& B, const Pages& P) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      int key = blk + 16 * t + col;
-      key = key < kmax ? key : kmax;
-      const bf16* kp = k_cache + (((size_t)P.k[t] * Hkv + kvh) * page + key % page) * D;
+      const bf16* kp = k_cache + (((size_t)P.k[t] * Hkv + kvh) * page + P.koff[t]) * D;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const int d0 = ks * 32 + kb * 8;
         B.a[t][ks].q = *reinterpret_cast<const uint4*>(kp + (d0 < D ? d0 : 0));
       }
     }
-    int k0 = blk + 4 * kb, k1 = blk + 16 + 4 * kb;
-    const int last = kmax & ~3;
-    k0 = k0 < last ? k0 : last;
-    k1 = k1 < last ? k1 : last;
-    const bf16* v0 = v_cache + ((size_t)P.v[0] * Hkv + kvh) * D * page + k0 % page;
-    const bf16* v1 = v_cache + ((size_t)P.v[1] * Hkv + kvh) * D * page + k1 % page;
+    const bf16* v0 = v_cache + ((size_t)P.v[0] * Hkv + kvh) * D * page + P.voff[0];
+    const bf16* v1 = v_cache + ((size_t)P.v[1] * Hkv + kvh) * D * page + P.voff[1];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       const size_t drow = (size_t)(dt * 16 + col) * page;
@@ -437,11 +467,10 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
     if (whole) {
 #pragma unroll
       for (int j = 0; j < PF_NT; ++j) {
-        float mx = fmaxf(fmaxf(fmaxf(S[j][0][0], S[j][0][1]), fmaxf(S[j][0][2], S[j][0][3])),
-                         fmaxf(fmaxf(S[j][1][0], S[j][1][1]), fmaxf(S[j][1][2], S[j][1][3])));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m[j], mx * scale_log2);
+        float mx = max_nn(max_nn(max_nn(S[j][0][0], S[j][0][1]), max_nn(S[j][0][2], S[j][0][3])),
+                         max_nn(max_nn(S[j][1][0], S[j][1][1]), max_nn(S[j][1][2], S[j][1][3])));
+        mx = quad_max(mx);
+        const float m_new = max_nn(m[j], mx * scale_log2);
         alpha[j] = fast_exp2(m[j] - m_new);
         m[j] = m_new;
 #pragma unroll
@@ -462,11 +491,10 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
           for (int i = 0; i < 4; ++i) {
             const int key = blk + 16 * t + 4 * kb + i;
             ok[t * 4 + i] = key >= lo && key <= hi;
-            mx = fmaxf(mx, ok[t * 4 + i] ? S[j][t][i] : -INFINITY);
+            mx = max_nn(mx, ok[t * 4 + i] ? S[j][t][i] : -INFINITY);
           }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m[j], mx * scale_log2);
+        mx = quad_max(mx);
+        const float m_new = max_nn(m[j], mx * scale_log2);
         // a query may see none of this block's keys (it lies before the block, or the block before its window)
         alpha[j] = m_new == -INFINITY ? 1.f : fast_exp2(m[j] - m_new);
         m[j] = m_new;
@@ -481,9 +509,8 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
     bool moved = false;
 #pragma unroll
     for (int j = 0; j < PF_NT; ++j) {
-      float rs = ((p[j][0] + p[j][1]) + (p[j][2] + p[j][3])) + ((p[j][4] + p[j][5]) + (p[j][6] + p[j][7]));
-      rs += __shfl_xor(rs, 16, 64);
-      rs += __shfl_xor(rs, 32, 64);
+      // l stays a per-lane partial sum (the lane's own keys); a query's four lanes are added at the end
+      const float rs = ((p[j][0] + p[j][1]) + (p[j][2] + p[j][3])) + ((p[j][4] + p[j][5]) + (p[j][6] + p[j][7]));
       l[j] = l[j] * alpha[j] + rs;
 #pragma unroll
       for (int e = 0; e < 4; ++e) pb[j].w[e] = pack_bf16(p[j][2 * e], p[j][2 * e + 1]);
@@ -504,23 +531,23 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
 
   KeyBlock b0, b1;
   Pages pg;
-  const int blk0 = kmin & ~(BLOCK_KEYS - 1);
   lookup_pages(pg, blk0);
-  load_block(b0, pg, blk0);
+  load_block(b0, pg);
   lookup_pages(pg, blk0 + BLOCK_KEYS);
   for (int blk = blk0; blk <= kmax; blk += 2 * BLOCK_KEYS) {
-    load_block(b1, pg, blk + BLOCK_KEYS);             // in flight while block 0 is computed
+    load_block(b1, pg);                               // in flight while block 0 is computed
     lookup_pages(pg, blk + 2 * BLOCK_KEYS);
     compute(b0, blk);
-    load_block(b0, pg, blk + 2 * BLOCK_KEYS);
+    load_block(b0, pg);
     lookup_pages(pg, blk + 3 * BLOCK_KEYS);
     if (blk + BLOCK_KEYS <= kmax) compute(b1, blk + BLOCK_KEYS);
   }
 
 #pragma unroll
   for (int j = 0; j < PF_NT; ++j) {
+    const float total = quad_sum(l[j]);
     if (!q_ok[j]) continue;
-    const float inv = 1.0f / l[j];
+    const float inv = 1.0f / total;
     bf16* op = out + ((size_t)qtok[j] * Hq + head[j]) * D + 4 * kb;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
