@@ -104,7 +104,7 @@ def measure_prefill(eng, tokens: int, seed: int):
     import torch
     from mini_inference_engine_amd import SamplingParams
     times = []
-    for rep in range(3):                      # the first run loads libraries and picks GEMM kernels
+    for rep in range(6):                      # the first run loads libraries and picks GEMM kernels
         p = prompts_of(1, tokens, eng.model_cfg.vocab_size, seed + rep)[0]
         eng.add_request(p, SamplingParams(max_tokens=1, ignore_eos=True))
         torch.cuda.synchronize()

@@ -99,11 +99,13 @@ class HipBackend(KernelBackend):
                 "mie_decode_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                                          c_int, c_void_p],
+                "mie_decode_block_keys": [],
+                "mie_attention_bf16_head_dim": [],
+            },
+            "prefill_attention_bf16": {
                 "mie_prefill_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                           c_void_p],
-                "mie_decode_block_keys": [],
-                "mie_attention_bf16_head_dim": [],
             },
         }.get(module, {})
         for name, argtypes in sig.items():
@@ -412,7 +414,7 @@ class HipBackend(KernelBackend):
                                ("row_position", step.row_position, step.num_rows)):
                 if t is None or t.dtype != torch.int32 or t.shape[0] < n or not t.is_contiguous():
                     raise ValueError(f"paged_attention: {name} must be contiguous int32 [{n}]")
-            lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))
+            lib = self.lib("prefill_attention_bf16", (f"-DHEAD_DIM={D}",))
             library.check(lib, lib.mie_prefill_attention(
                 _ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(bt), bt.shape[1],
                 _ptr(step.row_start), _ptr(step.row_position), step.num_decode_rows,

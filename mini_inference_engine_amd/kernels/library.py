@@ -24,9 +24,14 @@ import time
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 ARCH = "gfx950"
-MODULES = ("embed_norm", "rope_kv", "gemm", "attention", "sampling", "gemm_bf16", "attention_bf16")
+MODULES = ("embed_norm", "rope_kv", "gemm", "attention", "sampling", "gemm_bf16", "attention_bf16",
+           "prefill_attention_bf16")
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-fno-gpu-sanitize",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# Per module, beside FLAGS.  prefill_attention_bf16: matrix instructions keep their accumulators in
+# ordinary vector registers; otherwise the compiler parks the outputs in accumulation registers and copies
+# all of them back and forth around every key block for the sake of the (rare) rescaling.
+MODULE_FLAGS = {"prefill_attention_bf16": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 _loaded: dict = {}
 _lock = threading.Lock()
@@ -42,10 +47,10 @@ def available_modules() -> list[str]:
 
 def _digest(module: str, defines: tuple) -> str:
     h = hashlib.sha256()
-    for fn in (module + ".hip", "common.hpp"):
+    for fn in [module + ".hip"] + sorted(f for f in os.listdir(CSRC) if f.endswith(".hpp")):
         with open(os.path.join(CSRC, fn), "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS + [ARCH] + list(defines)).encode())
+    h.update(" ".join(FLAGS + MODULE_FLAGS.get(module, []) + [ARCH] + list(defines)).encode())
     return h.hexdigest()[:16]
 
 
@@ -101,7 +106,7 @@ def build(module: str, defines: tuple = (), verbose: bool = True) -> str:
         raise KernelLibraryError(f"no writable folder to build kernels in (tried {_build_dirs()})")
     out = os.path.join(out_dir, name)
     tmp = os.path.join(out_dir, f".{name}.{os.getpid()}.{threading.get_ident()}.tmp")
-    cmd = [_hipcc(), f"--offload-arch={ARCH}", *FLAGS, *defines, "-I", CSRC, src, "-o", tmp]
+    cmd = [_hipcc(), f"--offload-arch={ARCH}", *FLAGS, *MODULE_FLAGS.get(module, []), *defines, "-I", CSRC, src, "-o", tmp]
     env = dict(os.environ)
     env.setdefault("HOME", out_dir)        # hipcc's helpers want some HOME; an empty one is fine
     t0 = time.time()

@@ -1,6 +1,6 @@
 """Compile-time variants of the kernel modules that are built ahead of time.
 
-attention_bf16 is built once per head size.  The sizes listed here are those of the
+attention_bf16 and prefill_attention_bf16 are built once per head size.  The sizes listed here are those of the
 engine's benchmark shapes and tests; a model with another head size (any multiple of 16
 up to 256) gets its variant compiled at first use.
 """
@@ -9,4 +9,5 @@ HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
 
 VARIANTS = {
     "attention_bf16": [(f"-DHEAD_DIM={d}",) for d in HEAD_DIMS],
+    "prefill_attention_bf16": [(f"-DHEAD_DIM={d}",) for d in HEAD_DIMS],
 }
