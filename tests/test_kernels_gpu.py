@@ -514,7 +514,8 @@ def test_attention_window_edge(ops, dtype, window):
 
 
 @pytest.mark.parametrize("geom", [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 16), (6, 2, 80, 32), (8, 1, 128, 64),
-                                  (2, 2, 256, 16), (12, 4, 96, 16), (32, 4, 64, 16), (8, 8, 128, 16)])
+                                  (2, 2, 256, 16), (12, 4, 96, 16), (32, 4, 64, 16), (8, 8, 128, 16),
+                                  (20, 2, 64, 16), (16, 1, 256, 32), (6, 2, 64, 48), (5, 1, 32, 48)])
 @pytest.mark.parametrize("window", [None, 24])
 def test_prefill_attention_geometries(ops, geom, window):
     """The matrix-core prefill kernel: portions that start anywhere (page edges, mid page), tails that
