@@ -31,21 +31,14 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
   const int G = Hq / Hkv;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kb = lane >> 4;
-  const int pos = positions[b];
-  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
-  const int begin = (lo & ~(BLOCK_KEYS - 1)) + s * partition;
-  const int end = begin + partition < pos + 1 ? begin + partition : pos + 1;
   const int g = ht * 16 + col;
   const bool head_ok = g < G;
   const int head = kvh * G + (head_ok ? g : 0);
-
-  if (begin > pos) {          // this split lies beyond the row's keys (uniform over the workgroup)
-    if (num_splits > 1 && threadIdx.x < 16 && ht * 16 + (int)threadIdx.x < G)
-      lse_part[((size_t)b * Hq + kvh * G + ht * 16 + threadIdx.x) * num_splits + s] = -INFINITY;
-    return;
-  }
-
   const int* bt = block_tables + (size_t)b * max_blocks;
+
+  // Everything that can be asked for before the row's length is known is asked for first: the queries
+  // and, without a window, the first block of keys and values (pages are looked up by key index alone,
+  // clamped to the table; entries past the row's pages name the scratch page, whose contents are masked).
   Frag qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
@@ -53,49 +46,76 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
     qf[ks].q = make_uint4(0, 0, 0, 0);
     if (head_ok && d0 < D) qf[ks].q = *reinterpret_cast<const uint4*>(q + (size_t)b * q_stride + (size_t)head * D + d0);
   }
+  struct KeyBlock {
+    Frag a[2][KS];      // keys: 16 keys x 32 dims each
+    Frag va[DT];        // values: 16 dims x 32 keys each, in the order the probabilities sit in registers
+  };
+  const int last_page = max_blocks - 1;
+  auto load_block = [&](KeyBlock& B, int blk) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key = blk + 16 * t + col;
+      int pi = key / page;
+      pi = pi < last_page ? pi : last_page;
+      const bf16* kp = k_cache + (((size_t)bt[pi] * Hkv + kvh) * page + key % page) * D;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = ks * 32 + kb * 8;
+        B.a[t][ks].q = *reinterpret_cast<const uint4*>(kp + (d0 < D ? d0 : 0));
+      }
+    }
+    const int k0 = blk + 4 * kb, k1 = blk + 16 + 4 * kb;
+    int p0 = k0 / page, p1 = k1 / page;
+    p0 = p0 < last_page ? p0 : last_page;
+    p1 = p1 < last_page ? p1 : last_page;
+    const bf16* v0 = v_cache + ((size_t)bt[p0] * Hkv + kvh) * D * page + k0 % page;
+    const bf16* v1 = v_cache + ((size_t)bt[p1] * Hkv + kvh) * D * page + k1 % page;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const size_t drow = (size_t)(dt * 16 + col) * page;
+      B.va[dt].h[0] = *reinterpret_cast<const uint2*>(v0 + drow);
+      B.va[dt].h[1] = *reinterpret_cast<const uint2*>(v1 + drow);
+    }
+  };
+  constexpr bool AHEAD = D <= 128;          // two blocks in registers; larger heads have no room for it
+  KeyBlock b0, b1;
+  const int pos_raw = positions[b];
+  int begin0 = s * partition;               // the split's first key when there is no window
+  if (AHEAD && window <= 0) load_block(b0, begin0 + BLOCK_KEYS * wave);
+
+  const int pos = pos_raw;
+  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  const int begin = (lo & ~(BLOCK_KEYS - 1)) + s * partition;
+  const int end = begin + partition < pos + 1 ? begin + partition : pos + 1;
+
+  if (begin > pos) {          // this split lies beyond the row's keys (uniform over the workgroup)
+    if (num_splits > 1 && threadIdx.x < 16 && ht * 16 + (int)threadIdx.x < G)
+      lse_part[((size_t)b * Hq + kvh * G + ht * 16 + threadIdx.x) * num_splits + s] = -INFINITY;
+    return;
+  }
 
   float m = -INFINITY, l = 0.f;
   f32x4 O[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) O[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int blk = begin + BLOCK_KEYS * wave; blk < end; blk += BLOCK_KEYS * NW) {
+  auto compute = [&](KeyBlock& B, int blk) {
+    if (D % 32 != 0) {
+      // the last 32-dim step of the keys is half empty: its upper lanes were loaded from dim 0
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        if ((KS - 1) * 32 + kb * 8 >= D) B.a[t][KS - 1].q = make_uint4(0, 0, 0, 0);
+    }
     // ---- scores of 32 keys x 16 heads
     f32x4 S[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       S[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-      int key = blk + 16 * t + col;
-      key = key < pos ? key : pos;                      // never look up pages the row does not have
-      const int pg = bt[key / page];
-      const bf16* kp = k_cache + (((size_t)pg * Hkv + kvh) * page + key % page) * D;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int d0 = ks * 32 + kb * 8;
-        Frag a;
-        a.q = make_uint4(0, 0, 0, 0);
-        if (d0 < D) a.q = *reinterpret_cast<const uint4*>(kp + d0);
-        S[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[ks].v, S[t], 0, 0, 0);
-      }
+      for (int ks = 0; ks < KS; ++ks)
+        S[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(B.a[t][ks].v, qf[ks].v, S[t], 0, 0, 0);
     }
-    // ---- values of the same 32 keys, in the order the probabilities sit in registers
     const bool partial = blk + BLOCK_KEYS > pos + 1 || blk < lo;
-    Frag va[DT];
-    {
-      int k0 = blk + 4 * kb, k1 = blk + 16 + 4 * kb;
-      const int last = pos & ~3;
-      k0 = k0 < last ? k0 : last;
-      k1 = k1 < last ? k1 : last;
-      const int pg0 = bt[k0 / page], pg1 = bt[k1 / page];
-      const bf16* v0 = v_cache + ((size_t)pg0 * Hkv + kvh) * D * page + k0 % page;
-      const bf16* v1 = v_cache + ((size_t)pg1 * Hkv + kvh) * D * page + k1 % page;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const size_t drow = (size_t)(dt * 16 + col) * page;
-        va[dt].h[0] = *reinterpret_cast<const uint2*>(v0 + drow);
-        va[dt].h[1] = *reinterpret_cast<const uint2*>(v1 + drow);
-      }
-    }
     // ---- online softmax, one head per lane column
     float sv[8];
     bool ok[8];
@@ -132,16 +152,34 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          uint32_t w = va[dt].w[j];
+          uint32_t w = B.va[dt].w[j];
           if (!ok[2 * j]) w &= 0xFFFF0000u;
           if (!ok[2 * j + 1]) w &= 0x0000FFFFu;
-          va[dt].w[j] = w;
+          B.va[dt].w[j] = w;
         }
     }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       O[dt] *= alpha;
-      O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt].v, pb.v, O[dt], 0, 0, 0);
+      O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(B.va[dt].v, pb.v, O[dt], 0, 0, 0);
+    }
+  };
+
+  constexpr int STEP = BLOCK_KEYS * NW;     // keys from one block of a wave to its next
+  const int first = begin + BLOCK_KEYS * wave;
+  if (AHEAD) {
+    if (window > 0) load_block(b0, first);  // with a window the split's start had to wait for the row's length
+    const int part_end = begin + partition;   // nothing is asked for beyond the split's own keys
+    for (int blk = first; blk < end; blk += 2 * STEP) {
+      if (blk + STEP < part_end) load_block(b1, blk + STEP);           // in flight while block 0 is computed
+      compute(b0, blk);
+      if (blk + 2 * STEP < part_end) load_block(b0, blk + 2 * STEP);
+      if (blk + STEP < end) compute(b1, blk + STEP);
+    }
+  } else {
+    for (int blk = first; blk < end; blk += STEP) {
+      load_block(b0, blk);
+      compute(b0, blk);
     }
   }
 
