@@ -96,10 +96,7 @@ __global__ void __launch_bounds__(WAVES * 64)
 skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict__ W, long ldw, void* __restrict__ outv,
                    long ldo, int M, int N, int K, int up_offset, RopeArgs rope, NormArgs nf) {
   // k-steps per group of loads (two groups are in flight per wave)
-#ifndef SG_U_SCALE
-#define SG_U_SCALE 1
-#endif
-  constexpr int U = (MT == 1 ? 4 : (MT == 2 ? 2 : 1)) * SG_U_SCALE;
+  constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
   constexpr int SG_WAVES = WAVES;
   constexpr int SG_THREADS = WAVES * 64;
   constexpr int PER = (MT * 256 + SG_THREADS - 1) / SG_THREADS;   // results (m, n) a thread owns after the reduction
@@ -367,25 +364,16 @@ static int launch_waves(int waves, bool fused_norm, int epi, dim3 grid, hipStrea
   MIE_FAIL("skinny_gemm: %d waves", waves);
 }
 
-#ifdef SG_EXPERIMENT
-static int g_force_waves = 0;
-#endif
-
 // Waves a tile: the fewer tiles a product has, the more waves share one, so that enough loads are in
 // flight to fill the memory system (16 waves were measured slower than 8 at every shape).  Chosen from
 // the weight's shape alone, never from the batch.
-static int waves_for(int tiles, int K) {
-#ifdef SG_EXPERIMENT
-  if (g_force_waves) return g_force_waves;
-#endif
-  return tiles < 256 ? 8 : 4;
-}
+static int waves_for(int tiles) { return tiles < 256 ? 8 : 4; }
 
 static int launch_rows(int tiles, int epi, hipStream_t s, const bf16* X, long ldx, const bf16* W, long ldw, void* out,
                        long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope, const NormArgs* nf) {
   dim3 grid(tiles);
   const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  const int waves = waves_for(tiles, K);
+  const int waves = waves_for(tiles);
   NormArgs none = {};
   const NormArgs& n = nf ? *nf : none;
   if (MT == 1) return launch_waves<1>(waves, nf != nullptr, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n);
