@@ -3,7 +3,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048]
 
 A step is one decode step of the engine (schedule, batch, captured forward, sampling,
-bookkeeping: LLMEngine.step, the call a user's loop makes), after the method of the
+bookkeeping: LLMEngine.step, the call a user's loop makes; it starts a step and reads the tokens
+of the one before, so K calls between two synchronisations are K whole steps), after the method of the
 reference's benchmarks/bench_latency.py:33-49: prefill ``batch`` equal prompts, warm up,
 time K steps between device synchronisations.  Prints one JSON line:
   value     decoded tokens a second at ``batch`` (default 8) with contexts just below ``context``
@@ -95,7 +96,7 @@ def measure_decode(eng, batch: int, context: int, steps: int, warmup: int, seed:
     captured = eng.num_graph_steps - g0
     assert len(eng.scheduler.running) == batch, "a request ended inside the timed steps"
     mid_context = int(sum(s.num_tokens for s in eng.scheduler.running) / batch) - steps // 2
-    while eng.scheduler.has_work():
+    while eng.has_work():
         eng.step()
     return dt, captured, mid_context
 
@@ -109,7 +110,8 @@ def measure_prefill(eng, tokens: int, seed: int):
         eng.add_request(p, SamplingParams(max_tokens=1, ignore_eos=True))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        done = eng.step()
+        eng.step()
+        done = eng.drain()                    # the step just started is the one read
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         assert len(done) == 1 and done[0].num_computed == tokens, "the prompt did not run as one step"
@@ -172,7 +174,7 @@ def main() -> int:
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "global_batch": args.batch, "seq_len": args.context, "context_at_mid_run": main_r["context"],
                    "page_size": args.block_size, "captured_steps": main_r["captured"], "parallelism": "single GPU",
-                   "step": "LLMEngine.step: schedule + forward + sample"},
+                   "step": "LLMEngine.step: schedule + forward + sample, one step ahead of the token read-back"},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
     }

@@ -27,6 +27,7 @@ class EngineConfig:
     seed: int = 0                           # base of every request's sampling stream
     activation_reserve_bytes: int = 768 * 2**20
     poison_freed_pages: bool = False        # debugging: fill returned pages with NaN
+    run_ahead: bool = True                  # start a step before the host has read the tokens of the one before
 
     def __post_init__(self):
         if self.block_size < 16 or self.block_size % 16:

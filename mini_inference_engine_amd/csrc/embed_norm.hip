@@ -9,9 +9,14 @@
 
 template <typename TT>
 __global__ void embedding_kernel(const int* __restrict__ ids, const TT* __restrict__ table, float* __restrict__ out,
-                                 int width, int vocab) {
+                                 int width, int vocab, const int* __restrict__ taken_from,
+                                 const int* __restrict__ earlier_tokens) {
   const int t = blockIdx.x;
   int id = ids[t];
+  if (taken_from) {            // a token the host does not know yet: entry taken_from[t] of the tokens chosen last
+    const int j = taken_from[t];
+    if (j >= 0) id = earlier_tokens[j];
+  }
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // ids are validated on the host; never read outside
   const TT* src = table + (size_t)id * width;
   float* dst = out + (size_t)t * width;
@@ -135,15 +140,20 @@ add_rmsnorm_fast_kernel(const TX* __restrict__ x, float* __restrict__ stream, co
 
 MIE_EXPORT const char* embed_norm_last_error() { return g_mie_error; }
 
+// taken_from (or null) [tokens]: where >= 0, the token is earlier_tokens[taken_from[t]] instead of ids[t]
+// (a token chosen by the step before, which the host has not seen yet).
 MIE_EXPORT int mie_embedding(const int* ids, const void* table, int table_dtype, float* out, int tokens, int width,
-                             int vocab, hipStream_t stream) {
+                             int vocab, const int* taken_from, const int* earlier_tokens, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (width <= 0 || vocab <= 0) MIE_FAIL("embedding: width %d, vocab %d", width, vocab);
+  if (taken_from && !earlier_tokens) MIE_FAIL("embedding: taken_from without the tokens to take from");
   dim3 grid(tokens), block(256);
   if (table_dtype == MIE_F32)
-    hipLaunchKernelGGL(embedding_kernel<float>, grid, block, 0, stream, ids, (const float*)table, out, width, vocab);
+    hipLaunchKernelGGL(embedding_kernel<float>, grid, block, 0, stream, ids, (const float*)table, out, width, vocab,
+                       taken_from, earlier_tokens);
   else if (table_dtype == MIE_BF16)
-    hipLaunchKernelGGL(embedding_kernel<bf16>, grid, block, 0, stream, ids, (const bf16*)table, out, width, vocab);
+    hipLaunchKernelGGL(embedding_kernel<bf16>, grid, block, 0, stream, ids, (const bf16*)table, out, width, vocab,
+                       taken_from, earlier_tokens);
   else
     MIE_FAIL("embedding: table dtype code %d", table_dtype);
   MIE_CHECK_LAUNCH("embedding");

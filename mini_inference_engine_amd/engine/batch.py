@@ -24,6 +24,8 @@ class StepRow:
     tokens: Sequence[int]            # the tokens to run now
     start: int                       # position of tokens[0] = tokens of the request already in the cache
     want: Sequence[int] = ()         # offsets into ``tokens`` whose logits are wanted
+    taken_from: int = -1             # >= 0: the row's one token is that entry of the tokens the last step chose
+                                     # (still on the device); ``tokens`` then holds a placeholder
 
 
 @dataclass
@@ -48,6 +50,8 @@ class StepContext:
     row_context: torch.Tensor        # [rows] int32 keys visible after this step = position + length
     state_slots: torch.Tensor        # [rows] int32
     logit_rows: torch.Tensor         # [num_logits] int32 flat token positions, in the caller's order
+    taken_from: torch.Tensor | None = None      # [T] int32, see StepRow.taken_from; -1 where input_ids holds the token
+    earlier_tokens: torch.Tensor | None = None  # int32: the tokens the last step chose (set by the runner)
     groups: list = field(default_factory=list)
     page_size: int = 0
     max_row_tokens: int = 0          # longest row (host)
@@ -61,7 +65,7 @@ class StepArena:
     def __init__(self, max_tokens: int, max_rows: int, max_blocks: int, num_groups: int, device):
         self.max_tokens, self.max_rows, self.max_blocks, self.num_groups = max_tokens, max_rows, max_blocks, num_groups
         self.device = torch.device(device)
-        fields_ = [("input_ids", max_tokens), ("positions", max_tokens), ("token_row", max_tokens),
+        fields_ = [("input_ids", max_tokens), ("taken_from", max_tokens), ("positions", max_tokens), ("token_row", max_tokens),
                    ("logit_rows", max_tokens), ("row_start", max_rows + 1), ("row_position", max_rows),
                    ("row_context", max_rows), ("state_slots", max_rows)]
         for g in range(num_groups):
@@ -92,8 +96,6 @@ class StepArena:
         """One copy of everything before the block tables plus the used rows of the tables."""
         if self.dev is self.host:
             return
-        if self._copied is not None:
-            self._copied.synchronize()       # the pinned mirror was free to overwrite only after this
         end = self.tables_begin
         self.dev[:end].copy_(self.host[:end], non_blocking=True)
         for g in range(self.num_groups):
@@ -119,6 +121,7 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
     """Flatten ``rows`` into ``arena``.  ``pad_rows_to`` adds scratch rows (one token at
     position 0, page 0, slot 0) up to a captured batch size.  ``want_all`` asks for the logits
     of every token in flat order (what a captured step produces) instead of the rows' wants."""
+    arena.wait_uploaded()           # the last step's copy may still be reading the host mirror
     order = order_rows(rows)
     n_rows = len(rows)
     lens = np.fromiter((len(rows[i].tokens) for i in order), dtype=np.int64, count=n_rows)
@@ -148,6 +151,8 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
         raise ValueError(f"a row needs {blocks_needed} pages; the arena holds {arena.max_blocks} per row")
 
     ids = arena.host_view("input_ids")
+    taken = arena.host_view("taken_from")
+    taken[:T] = -1
     slots_state = arena.host_view("state_slots")
     new_row_of = {}
     for r, i in enumerate(src):
@@ -156,7 +161,13 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
             ids[a:b] = 0
             slots_state[r] = 0
         else:
-            ids[a:b] = rows[i].tokens
+            if rows[i].taken_from >= 0:
+                if b - a != 1:
+                    raise ValueError("only a single-token row can take its token from the last step's choices")
+                ids[a] = 0
+                taken[a] = rows[i].taken_from
+            else:
+                ids[a:b] = rows[i].tokens
             slots_state[r] = rows[i].cache.state_slot
             new_row_of[i] = r
     arena.host_view("positions")[:T] = positions
@@ -195,7 +206,8 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
     arena.upload(total_rows)
     step = StepContext(
         num_tokens=T, num_rows=total_rows, num_decode_rows=num_decode, num_logits=R,
-        input_ids=arena.dev_view("input_ids", T), positions=arena.dev_view("positions", T),
+        input_ids=arena.dev_view("input_ids", T), taken_from=arena.dev_view("taken_from", T),
+        positions=arena.dev_view("positions", T),
         token_row=arena.dev_view("token_row", T), row_start=arena.dev_view("row_start", total_rows + 1),
         row_position=arena.dev_view("row_position", total_rows), row_context=arena.dev_view("row_context", total_rows),
         state_slots=arena.dev_view("state_slots", total_rows), logit_rows=arena.dev_view("logit_rows", R),

@@ -20,7 +20,7 @@ from ..sampling import Sampler, SamplingParams
 from .batch import StepRow
 from .runner import ModelRunner, parse_dtype
 from .scheduler import Scheduler
-from .sequence import Sequence
+from .sequence import PENDING, Sequence, Status
 
 
 @dataclass
@@ -31,6 +31,15 @@ class RequestOutput:
     text: str | None
     ttft: float | None          # seconds from arrival to the first generated token
     latency: float | None       # seconds from arrival to the end
+
+
+@dataclass
+class _StepInFlight:
+    """A step that was started and whose chosen tokens the host has not read."""
+    seqs: list                  # the requests a token is being chosen for, in sampling order
+    places: list                # where in each request's token list that token goes
+    chosen: object              # sampling.ChosenTokens, or None if no row wanted a token
+    index_of: dict              # request -> its entry among the chosen tokens (for the next step's rows)
 
 
 class LLMEngine:
@@ -53,7 +62,8 @@ class LLMEngine:
         if cfg.poison_freed_pages:
             self.cache.on_release = self.runner.storage.poison_pages
         self.scheduler = Scheduler(self.cfg, self.cache)
-        self.sampler = Sampler(self.runner.ops, self.runner.device, cfg.max_num_seqs)
+        self.sampler = Sampler(self.runner.ops, self.runner.device, cfg.max_num_seqs, out=self.runner.chosen_tokens)
+        self._in_flight = None             # the step whose tokens the host has not read yet
         self.eos_token_id = self.runner.model.spec.eos_token_id
         if verbose:
             print(f"[mini_inference_engine_amd] cache: {self.runner.num_pages} pages x {cfg.block_size} tokens "
@@ -96,16 +106,50 @@ class LLMEngine:
         return seq
 
     # ------------------------------------------------------------------- step
+    def has_work(self) -> bool:
+        return self._in_flight is not None or self.scheduler.has_work()
+
     def step(self) -> list[Sequence]:
-        """One scheduling + forward + sampling step.  Returns the requests that finished."""
+        """Starts one step (schedule, forward, sampling) and then reads the tokens of the step before it,
+        which ran on the device while this one was prepared.  Returns the requests which that earlier step
+        finished.  With ``run_ahead`` off, the step started is also the one read.
+
+        Running one step ahead: a request's next row is scheduled before its last token is known to the
+        host; the device takes the token from where the sampling kernel left it.  What does not depend on
+        the token's value (positions, pages, the end by max_tokens or length) is decided at once; an end
+        by the stop token is seen one step late, and the row already started for that request is dropped."""
+        started = self._start()
+        if not self.cfg.run_ahead:
+            return self._finish_step(started) if started is not None else []
+        finished = self._finish_step(self._in_flight) if self._in_flight is not None else []
+        self._in_flight = started
+        return finished
+
+    def drain(self) -> list[Sequence]:
+        """Reads the tokens of the step that is still on its way, if any, without starting another."""
+        if self._in_flight is None:
+            return []
+        finished = self._finish_step(self._in_flight)
+        self._in_flight = None
+        return finished
+
+    def _start(self):
         batch = self.scheduler.schedule()
         if not batch:
-            return []
+            return None
+        taken = self._in_flight.index_of if self._in_flight is not None else {}
         rows, sample_seqs = [], []
         for seq, n in batch:
             nc = seq.num_computed
             last = nc + n == seq.num_tokens
-            rows.append(StepRow(seq.cache, seq.token_ids[nc:nc + n], nc, [n - 1] if last else []))
+            tokens = seq.token_ids[nc:nc + n]
+            source = -1
+            if tokens[-1] == PENDING:
+                # only ever the one token the step in flight is choosing for this request
+                if n != 1 or seq not in taken:
+                    raise RuntimeError(f"request {seq.seq_id}: a token not yet known in a row of {n}")
+                tokens, source = [0], taken[seq]
+            rows.append(StepRow(seq.cache, tokens, nc, [n - 1] if last else [], taken_from=source))
             if last:
                 sample_seqs.append(seq)
 
@@ -115,29 +159,46 @@ class LLMEngine:
             self.num_graph_steps += 1
         else:
             logits = self.runner.forward_step(rows)
+        self.num_steps += 1
 
-        new_tokens = []
+        chosen = None
         if sample_seqs:
-            new_tokens = self.sampler.sample(
+            chosen = self.sampler.sample_async(
                 logits, [s.params.temperature for s in sample_seqs], [s.seed for s in sample_seqs],
                 [s.num_output_tokens for s in sample_seqs])
 
-        self.num_steps += 1
+        # what is certain whatever the tokens turn out to be
         for seq, n in batch:
             self.scheduler.advance(seq, n)
+        places = []
+        for seq in sample_seqs:
+            places.append(seq.num_tokens)
+            seq.token_ids.append(PENDING)
+            if seq.num_output_tokens >= seq.params.max_tokens or seq.num_tokens >= self.cfg.max_model_len:
+                seq.ending = True              # its last token is on its way: not to be scheduled again
+        return _StepInFlight(sample_seqs, places, chosen, {s: j for j, s in enumerate(sample_seqs)})
+
+    def _finish_step(self, st) -> list[Sequence]:
+        tokens = st.chosen.tolist() if st.chosen is not None else []
         now = time.perf_counter()
         finished = []
-        for seq, tok in zip(sample_seqs, new_tokens):
-            seq.token_ids.append(tok)
+        for seq, place, tok in zip(st.seqs, st.places, tokens):
+            if seq.status is Status.FINISHED:
+                continue                       # ended by its stop token a step ago; this row was one too many
+            seq.token_ids[place] = tok
             if seq.first_token_time is None:
                 seq.first_token_time = now
-            done = (seq.num_output_tokens >= seq.params.max_tokens
-                    or seq.num_tokens >= self.cfg.max_model_len
-                    or (tok == self.eos_token_id and not seq.params.ignore_eos))
-            if done:
-                seq.finish_time = now
+            stopped = tok == self.eos_token_id and not seq.params.ignore_eos
+            if not (stopped or (seq.ending and place == seq.num_tokens - 1)):
+                continue
+            del seq.token_ids[place + 1:]      # a placeholder of the row started meanwhile, if any
+            seq.finish_time = now
+            if seq.status is Status.RUNNING:
                 self.scheduler.finish(seq)
-                finished.append(seq)
+            else:                              # preempted while its last token was on its way
+                self.scheduler.waiting.remove(seq)
+                seq.status = Status.FINISHED
+            finished.append(seq)
         return finished
 
     # --------------------------------------------------------------- offline
@@ -148,7 +209,7 @@ class LLMEngine:
         if len(params) != len(prompts):
             raise ValueError(f"{len(prompts)} prompts but {len(params)} sampling params")
         seqs = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
-        while self.scheduler.has_work():
+        while self.has_work():
             self.step()
         outs = []
         for s in seqs:

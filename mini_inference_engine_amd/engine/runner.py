@@ -79,6 +79,9 @@ class ModelRunner:
         self.model.attach_cache(self.storage)
         self.arena = StepArena(max_step_tokens, max_rows, self.max_blocks, n_groups, self.device)
         self.vocab_size = spec.vocab_size
+        # The tokens the last step chose, at a fixed address: the next step's rows may take their token
+        # from here on the device (StepRow.taken_from) before the host has seen it.
+        self.chosen_tokens = torch.zeros(max(1, max_rows), dtype=torch.int32, device=self.device)
 
     # ------------------------------------------------------------------ steps
     def build(self, rows: list[StepRow], **kw):
@@ -86,7 +89,11 @@ class ModelRunner:
             if r.start + len(r.tokens) > self.max_model_len:
                 raise ValueError(f"a row reaches position {r.start + len(r.tokens)}, beyond max_model_len "
                                  f"{self.max_model_len}")
-        return build_step(rows, self.arena, self.page_size, **kw)
+            if r.taken_from >= self.chosen_tokens.numel():
+                raise ValueError(f"a row takes its token from entry {r.taken_from} of {self.chosen_tokens.numel()}")
+        step = build_step(rows, self.arena, self.page_size, **kw)
+        step.earlier_tokens = self.chosen_tokens
+        return step
 
     @torch.inference_mode()
     def forward_step(self, rows: list[StepRow]) -> torch.Tensor | None:

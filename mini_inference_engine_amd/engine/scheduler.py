@@ -80,7 +80,7 @@ class Scheduler:
         preemptions_before = self.num_preemptions
 
         for seq in list(self.running):
-            if seq.status is not Status.RUNNING or seq.num_new_tokens != 1:
+            if seq.status is not Status.RUNNING or seq.num_new_tokens != 1 or seq.ending:
                 continue
             if budget == 0:
                 break
@@ -89,7 +89,7 @@ class Scheduler:
                 budget -= 1
 
         for seq in list(self.running):
-            if seq.status is not Status.RUNNING or seq.num_new_tokens <= 1 or budget == 0:
+            if seq.status is not Status.RUNNING or seq.num_new_tokens <= 1 or budget == 0 or seq.ending:
                 continue
             n = min(seq.num_new_tokens, budget)
             if not self.cfg.enable_chunked_prefill and n < seq.num_new_tokens:
@@ -122,7 +122,8 @@ class Scheduler:
             prefills.append((seq, n))
             budget -= n
 
-        if not decodes and not prefills and self.has_work():
+        if not decodes and not prefills and self.has_work() and not any(s.ending for s in self.running):
+            # (a request whose last token is on its way will make room when it ends)
             raise RequestTooLarge("nothing can be scheduled although requests are waiting: "
                                   "the head of the queue does not fit the cache or the budget")
         return decodes + prefills

@@ -10,6 +10,8 @@ from ..sampling.params import SamplingParams
 
 _ids = itertools.count()
 
+PENDING = -1     # stands in a request's token list for a token that is being chosen on the device
+
 
 class Status(enum.Enum):
     WAITING = 0
@@ -29,6 +31,7 @@ class Sequence:
         self.num_computed = 0            # tokens whose keys and values are in the cache
         self.cache = None                # cache.RequestCache while running
         self.status = Status.WAITING
+        self.ending = False              # its last token is on its way (max_tokens or length): schedule no more
         self.num_preemptions = 0
         self.arrival_time = time.perf_counter()
         self.first_token_time: float | None = None

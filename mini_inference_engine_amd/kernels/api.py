@@ -53,8 +53,10 @@ class KernelBackend:
     name = "?"
     act_dtype = None
 
-    def embedding(self, ids, table):
-        """stream[t, :] = float(table[ids[t], :]) -> [T, width] float32."""
+    def embedding(self, ids, table, taken_from=None, earlier_tokens=None):
+        """stream[t, :] = float(table[ids[t], :]) -> [T, width] float32.  With ``taken_from`` (int32 [T]):
+        where it is >= 0 the token is ``earlier_tokens[taken_from[t]]`` instead of ``ids[t]`` (a token the
+        step before chose, read on the device because the host has not seen it yet)."""
         raise NotImplementedError
 
     def add_rmsnorm(self, x, residual, weight, eps, out_dtype=None, rows=None):
@@ -103,7 +105,7 @@ class KernelBackend:
         qkv (row stride qkv.stride(0)).  Returns [T, Hq * D] in act_dtype."""
         raise NotImplementedError
 
-    def sample(self, logits, temperatures, seeds, counters):
+    def sample(self, logits, temperatures, seeds, counters, out=None):
         """Per row: argmax(logits) if temperature == 0, else argmax(logits / temperature + g)
-        with Gumbel noise g from (seed, counter, vocabulary index).  -> [R] int32."""
+        with Gumbel noise g from (seed, counter, vocabulary index).  -> [R] int32 (``out`` if given)."""
         raise NotImplementedError

@@ -65,7 +65,7 @@ class HipBackend(KernelBackend):
     def _declare(module: str, lib) -> None:
         sig = {
             "embed_norm": {
-                "mie_embedding": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+                "mie_embedding": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
                 "mie_add_rmsnorm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                                     c_int, c_float, c_void_p],
             },
@@ -122,17 +122,21 @@ class HipBackend(KernelBackend):
                 raise ValueError(f"tensor on {t.device}; the kernels take GPU tensors only")
 
     # ----------------------------------------------------------------- ops
-    def embedding(self, ids, table):
-        self._on_device(ids, table)
+    def embedding(self, ids, table, taken_from=None, earlier_tokens=None):
+        self._on_device(ids, table, taken_from, earlier_tokens)
         if ids.dtype != torch.int32 or ids.dim() != 1 or not ids.is_contiguous():
             raise ValueError("embedding: ids must be contiguous int32 [T]")
+        if taken_from is not None:
+            if earlier_tokens is None or taken_from.dtype != torch.int32 or earlier_tokens.dtype != torch.int32 \
+                    or taken_from.shape != ids.shape or not taken_from.is_contiguous() or not earlier_tokens.is_contiguous():
+                raise ValueError("embedding: taken_from must be contiguous int32 [T] beside int32 earlier_tokens")
         if table.dim() != 2 or not table.is_contiguous():
             raise ValueError("embedding: table must be contiguous [vocab, width]")
         T, (V, W) = ids.shape[0], table.shape
         out = torch.empty((T, W), dtype=torch.float32, device=table.device)
         lib = self.lib("embed_norm")
         library.check(lib, lib.mie_embedding(_ptr(ids), _ptr(table), _code(table.dtype), _ptr(out), T, W, V,
-                                             self._stream()))
+                                             _ptr(taken_from), _ptr(earlier_tokens), self._stream()))
         return out
 
     def add_rmsnorm(self, x, residual, weight, eps, out_dtype=None, rows=None):
@@ -431,8 +435,8 @@ class HipBackend(KernelBackend):
                 T - done, Hq, Hkv, D, page, float(scale), int(window or 0), self._stream()))
         return out
 
-    def sample(self, logits, temperatures, seeds, counters):
-        self._on_device(logits, temperatures, seeds, counters)
+    def sample(self, logits, temperatures, seeds, counters, out=None):
+        self._on_device(logits, temperatures, seeds, counters, out)
         if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
             raise ValueError("sample: logits must be float32 [rows, vocab] with unit inner stride")
         R, V = logits.shape
@@ -440,7 +444,10 @@ class HipBackend(KernelBackend):
             raise ValueError("sample: temperatures float32, seeds int64, counters int32")
         if not (temperatures.shape[0] == seeds.shape[0] == counters.shape[0] == R):
             raise ValueError("sample: one temperature, seed and counter per row")
-        out = torch.empty(R, dtype=torch.int32, device=logits.device)
+        if out is None:
+            out = torch.empty(R, dtype=torch.int32, device=logits.device)
+        elif out.dtype != torch.int32 or tuple(out.shape) != (R,) or not out.is_contiguous():
+            raise ValueError(f"sample: out must be contiguous int32 [{R}]")
         lib = self.lib("sampling")
         library.check(lib, lib.mie_sample(_ptr(logits), logits.stride(0), _ptr(temperatures), _ptr(seeds),
                                           _ptr(counters), _ptr(out), R, V, self._stream()))

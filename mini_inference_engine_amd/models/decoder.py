@@ -103,7 +103,7 @@ class Decoder:
         """Runs exactly the tokens of ``step`` and returns logits [wanted, vocab] in
         32-bit for ``step.logit_rows`` (flat token positions)."""
         spec = self.spec
-        residual = spec.embedding.forward(step.input_ids)
+        residual = spec.embedding.forward(step.input_ids, step.taken_from, step.earlier_tokens)
         h = None
         last = len(spec.schedule) - 1
         for e, (call, binding) in enumerate(zip(spec.schedule, self.bindings)):

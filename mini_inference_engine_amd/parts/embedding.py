@@ -21,8 +21,9 @@ class Embedding(Part):
     def params(self):
         return [ParamSpec.single("weight", self.weight_name, (self.vocab_size, self.width))]
 
-    def forward(self, ids):
-        return self.ops.embedding(ids, self.weight)
+    def forward(self, ids, taken_from=None, earlier_tokens=None):
+        """``taken_from`` / ``earlier_tokens``: see KernelBackend.embedding (tokens still on the device)."""
+        return self.ops.embedding(ids, self.weight, taken_from, earlier_tokens)
 
 
 class LMHead(Part):

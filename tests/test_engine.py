@@ -110,6 +110,53 @@ def test_eos_stops_and_stays(tiny_models):
     assert out[0].output_ids == toks[:stop + 1], "generation ends with the stop token, which stays in the output"
 
 
+def test_running_a_step_ahead_changes_no_token(tiny_models):
+    """A step is started before the host has read the tokens of the one before (the device hands them on);
+    stop tokens are then seen a step late.  Tokens, ends and the cache's books must be what they are when
+    every step is read before the next starts: mixed lengths, a small budget, stop tokens, few pages."""
+    m = tiny_models["B"]
+    prompts = prompts_for(m, [3, 25, 9, 40, 14, 1], seed=12)
+    free_run = engine(m, "cpu", "float32", num_blocks=40, max_num_seqs=6, run_ahead=False).generate(
+        prompts, SamplingParams(max_tokens=30, ignore_eos=True))
+    stop = free_run[2].output_ids[5]           # a token some request produces early: ends by stop token happen
+    params = [SamplingParams(max_tokens=30 - 3 * i, temperature=0.7 if i % 2 else 0.0, seed=50 + i) for i in range(6)]
+    results = {}
+    for ahead in (False, True):
+        for blocks in (40, 9):                 # roomy, and so tight that requests are preempted
+            eng = engine(m, "cpu", "float32", num_blocks=blocks, max_num_seqs=6, max_num_batched_tokens=24,
+                         run_ahead=ahead)
+            eng.eos_token_id = stop
+            outs = eng.generate(prompts, params)
+            eng.cache.check()
+            assert not eng.cache.live and not eng.has_work()
+            results[ahead, blocks] = [o.output_ids for o in outs]
+            if blocks == 9:
+                assert eng.scheduler.num_preemptions > 0, "the preemption path was not exercised"
+    assert any(ids and ids[-1] == stop and len(ids) < 12 for ids in results[False, 40]), "no request ended by the stop token"
+    assert results[True, 40] == results[False, 40]
+    assert results[True, 9] == results[False, 40] == results[False, 9]
+    for ids, sp in zip(results[True, 40], params):
+        assert len(ids) <= sp.max_tokens and -1 not in ids
+
+
+def test_step_returns_what_the_step_before_finished(tiny_models):
+    m = tiny_models["A"]
+    eng = engine(m, "cpu", "float32", num_blocks=16)
+    seq = eng.add_request(prompts_for(m, [6], seed=3)[0], SamplingParams(max_tokens=2, ignore_eos=True))
+    assert eng.step() == [] and eng.has_work()             # prompt started, its token not read yet
+    assert eng.step() == [] and seq.num_output_tokens == 2 and seq.token_ids[-1] == -1
+    assert eng.step() == [seq] and not eng.has_work()      # nothing to start; the last token is read
+    assert -1 not in seq.token_ids and len(seq.output_ids) == 2
+    eng2 = engine(m, "cpu", "float32", num_blocks=16)
+    seq2 = eng2.add_request(seq.token_ids[:6], SamplingParams(max_tokens=2, ignore_eos=True))
+    eng2.step()
+    assert eng2.drain() == [] and seq2.num_output_tokens == 1 and seq2.token_ids[-1] >= 0
+    assert eng2.drain() == []
+    while eng2.has_work():
+        eng2.step()
+    assert seq2.output_ids == seq.output_ids
+
+
 def test_entry_point_argument_errors(tiny_models):
     m = tiny_models["A"]
     eng = engine(m, "cpu", "float32", num_blocks=16)

@@ -131,8 +131,10 @@ class TorchBackend(KernelBackend):
     def _count(self, name):
         self.calls[name] = self.calls.get(name, 0) + 1
 
-    def embedding(self, ids, table):
+    def embedding(self, ids, table, taken_from=None, earlier_tokens=None):
         self._count("embedding")
+        if taken_from is not None:
+            ids = torch.where(taken_from >= 0, earlier_tokens[taken_from.clamp(min=0).long()], ids)
         return ref_embedding(ids, table)
 
     def add_rmsnorm(self, x, residual, weight, eps, out_dtype=None, rows=None):
@@ -170,6 +172,10 @@ class TorchBackend(KernelBackend):
         return ref_paged_attention(qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group.block_tables,
                                    step.token_row, step.positions, scale, window, self.act_dtype)
 
-    def sample(self, logits, temperatures, seeds, counters):
+    def sample(self, logits, temperatures, seeds, counters, out=None):
         self._count("sample")
-        return ref_sample(logits, temperatures, seeds, counters)
+        tokens = ref_sample(logits, temperatures, seeds, counters)
+        if out is None:
+            return tokens
+        out.copy_(tokens)
+        return out
