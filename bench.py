@@ -8,7 +8,8 @@ of the one before, so K calls between two synchronisations are K whole steps), a
 reference's benchmarks/bench_latency.py:33-49: prefill ``batch`` equal prompts, warm up,
 time K steps between device synchronisations.  Prints one JSON line:
   value     decoded tokens a second at ``batch`` (default 8) with contexts just below ``context``
-  points    the same at batch 1 and 64
+  points    the same at batch 1 and 64; output and total tokens a second of the reference's mixed
+            end-to-end workload (256 requests at once, prompts of 128..512 and outputs of 64..512 tokens)
   prefill   one 2,048-token prompt in one step: tokens a second, and flops / time / peak
   roofline  bytes a decode step must read (weights once + live cache) / time, against HBM peak
 Peaks: MI355X HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
@@ -118,6 +119,40 @@ def measure_prefill(eng, tokens: int, seed: int):
     return min(times[1:])
 
 
+def measure_mixed(cfg, weights, dtype, requests: int, seed: int, use_graphs: bool):
+    """The reference's end-to-end workload (benchmarks/bench_throughput.py:34-44 there): ``requests``
+    requests at once, prompt lengths uniform in [128, 512], output lengths uniform in [64, 512], stop
+    token ignored, up to 256 running; output tokens a second over the whole run."""
+    import random
+    import torch
+    from mini_inference_engine_amd import LLMEngine, SamplingParams
+    from mini_inference_engine_amd.config import EngineConfig
+    rng = random.Random(seed)
+    work = []
+    for _ in range(requests):
+        p, o = rng.randint(128, 512), rng.randint(64, 512)
+        work.append(([rng.randrange(3, cfg.vocab_size) for _ in range(p)], o))
+    ecfg = EngineConfig(max_num_seqs=256, max_num_batched_tokens=2048, max_model_len=1024,
+                        num_blocks=256 * 64 + 65, use_hip_graphs=use_graphs)
+    eng = LLMEngine(cfg, ecfg, dtype=dtype, verbose=False, weights=weights)
+    best = None
+    for rep in range(2):                      # the first run loads libraries and picks GEMM kernels
+        for ids, o in work:
+            eng.add_request(ids, SamplingParams(max_tokens=o, ignore_eos=True))
+        s0 = eng.num_steps
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while eng.has_work():
+            eng.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        best = (dt, eng.num_steps - s0)
+    out_tokens = sum(o for _, o in work)
+    all_tokens = out_tokens + sum(len(i) for i, _ in work)
+    return {"output_tok_s": round(out_tokens / best[0], 1), "total_tok_s": round(all_tokens / best[0], 1),
+            "seconds": round(best[0], 3), "steps": best[1], "preemptions": eng.scheduler.num_preemptions}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -153,7 +188,6 @@ def main() -> int:
                         max_model_len=args.context, num_blocks=pages, use_hip_graphs=not args.no_graphs,
                         graph_batch_sizes=tuple(batches))
     eng = LLMEngine(cfg, ecfg, dtype=dtype, verbose=False, weights=weights)
-    del weights
 
     results = {}
     for b in batches:
@@ -184,6 +218,12 @@ def main() -> int:
         n = 2048 if args.context >= 2048 else args.context
         line["prefill"] = {"value": round(n / t, 1), "tokens": n, "ms": round(t * 1e3, 3),
                            "frac": round(prefill_flops(cfg, n) / t / FLOP_PEAK[args.dtype], 4)}
+        if cfg.num_hidden_layers == full_layers and args.context >= 1024:
+            del eng
+            torch.cuda.empty_cache()
+            mixed = measure_mixed(cfg, weights, dtype, 256, 0, not args.no_graphs)
+            line["points"]["mixed_256_requests_output_tok_s"] = mixed["output_tok_s"]
+            line["points"]["mixed_256_requests_total_tok_s"] = mixed["total_tok_s"]
     print(json.dumps(line), flush=True)
     return 0
 
