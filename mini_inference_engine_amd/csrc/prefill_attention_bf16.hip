@@ -8,25 +8,33 @@
 // products as above with "head" replaced by "query": S^T[key, query] = K . Q^T and
 // O^T[d, query] += V^T . P^T, so softmax state is again one value per lane (its query).
 //
-// A workgroup of 4 waves serves one kv head and one stretch of 16 QT queries of a row; its waves own
-// PF_NT tiles each (16 queries x 1 head; hpw heads by qpw query tiles), waves_h of them side by side
-// over the heads of the group and 4 / waves_h over the queries.  All of them need the same keys: a
-// block of 32 keys and values is brought into the LDS once by the whole workgroup (two buffers, the
-// next block's loads in flight while the current one is computed, its pages looked up one block
-// earlier still), in rows padded so that the fragment reads of the matrix instructions meet no bank
-// conflict.  Work per stretch grows with its place in the row (causal), so a workgroup takes stretch
-// NS - 1 - i and then stretch i: every workgroup of a row has the same number of blocks to do.
+// A workgroup of PF_WAVES waves serves one kv head and one stretch of 16 QT queries of a row; its waves
+// own PF_NT tiles each (16 queries x 1 head; hpw heads by qpw query tiles), waves_h of them side by side
+// over the heads of the group and PF_WAVES / waves_h over the queries.  Eight waves of one tile keep two
+// waves on every SIMD: the kernel is bound by the number of vector instructions it issues (the softmax;
+// head size 64 gives the matrix unit little to do per score), and one wave's waits are the other's turn.
+// All waves need the same keys: a block of 32 keys and values is brought into the LDS once by the first
+// four waves (two LDS buffers and two sets of registers: block i + 1 waits in registers while block i is
+// computed, block i + 2 is on its way, the pages of block i + 3 are looked up), in rows padded so that
+// the fragment reads of the matrix instructions meet no bank conflict, values already in the key order
+// the second product wants.  Work per stretch grows with its place in the row (causal), so a workgroup
+// takes stretch NS - 1 - i and then stretch i: every workgroup of a row has the same number of blocks.
 // A block every query of a wave sees whole takes a path without masks; the running maximum m is kept
 // in units of scale * log2(e); l is a per-lane partial sum, joined over a query's four lanes at the end.
-constexpr int PF_NT = D <= 128 ? 2 : 1;
+// Timed alone (one row of 2,048 tokens, 32/4 heads of 64): 61 us, of which about 16 the softmax's vector
+// instructions, 14 the fragment reads from the LDS, 10 the matrix instructions, the rest bringing blocks in.
+constexpr int PF_WAVES = 8;                         // waves a workgroup
+constexpr int PF_NT = 1;                            // tiles a wave owns
+constexpr int PF_THREADS = PF_WAVES * 64;
 constexpr int PF_KROW = 2 * D + 16;                 // bytes of a key row in the LDS
 constexpr int PF_VROW = 2 * BLOCK_KEYS + 16;        // bytes of a value row (one dim, 32 keys) in the LDS
 constexpr int PF_KBYTES = BLOCK_KEYS * PF_KROW;
 constexpr int PF_BUF = PF_KBYTES + D * PF_VROW;     // one buffer: keys, then values
-constexpr int PF_PIECES = 4 * D;                    // 16-byte pieces of a block's keys (and of its values)
-constexpr int PF_PPT = (PF_PIECES + 255) / 256;     // pieces of each a thread carries
+constexpr int PF_PIECES = 4 * D;                    // 32-byte pieces of a block: 2 D of its keys, then 2 D of its values
+constexpr int PF_COPIERS = 256;                     // threads that bring a block in (the first four waves)
+constexpr int PF_PPT = (PF_PIECES + PF_COPIERS - 1) / PF_COPIERS;       // pieces such a thread carries
 
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(PF_THREADS)
 prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* __restrict__ k_cache,
                          const bf16* __restrict__ v_cache, bf16* __restrict__ out,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ row_start,
@@ -35,7 +43,7 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
   extern __shared__ __align__(16) unsigned char pf_lds[];
   const int row = first_row + blockIdx.y;
   const int G = Hq / Hkv;
-  const int qpw = PF_NT / hpw, waves_q = 4 / waves_h, QT = waves_q * qpw;
+  const int qpw = PF_NT / hpw, waves_q = PF_WAVES / waves_h, QT = waves_q * qpw;
   const int head_chunks = (G + hpw * waves_h - 1) / (hpw * waves_h);
   const int kvh = blockIdx.z / head_chunks, hc = blockIdx.z - kvh * head_chunks;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -98,18 +106,22 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
       for (int dt = 0; dt < DT; ++dt) O[j][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // ---- bringing a block into the LDS: piece c of the keys is 8 dims of one key, piece c of the values
-    // 8 keys of one dim.  Where the pieces lie (page and place in it) is found by walking the block table:
-    // [walk_start, walk_start + page) is the page of the block looked up last, and a key at most 31 past
-    // a block's start lies at most two pages on.  Addresses are clamped to the row's own keys.
+    // ---- bringing a block into the LDS, by the first PF_COPIERS threads (a SIMD then carries one wave that
+    // copies and one that does not): a piece is 32 bytes, 16 dims of one key or 16 keys of one dim, so one
+    // page look-up and one address serve two loads.  Where a piece lies (page and place in it) is found by
+    // walking the block table: [walk_start, walk_start + page) is the page of the block looked up last, and
+    // a key at most 31 past a block's start lies at most two pages on.  Addresses are clamped to the row's
+    // own keys.
     struct Where {
-      int kpg[PF_PPT], koff[PF_PPT], vpg[PF_PPT], voff[PF_PPT];
+      int pg[PF_PPT], off[PF_PPT];
     };
     struct Pieces {
-      uint4 k[PF_PPT], v[PF_PPT];
+      uint4 lo[PF_PPT], hi[PF_PPT];
     };
+    const bool copier = tid < PF_COPIERS;
     int walk_idx = blk0 / page, walk_start = walk_idx * page;
     auto lookup = [&](Where& Wh, int blk) {
+      if (!copier) return;
       blk = blk < last_blk ? blk : last_blk;           // beyond the last block: the last one again
       while (blk >= walk_start + page) {
         walk_start += page;
@@ -117,50 +129,65 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
       }
 #pragma unroll
       for (int i = 0; i < PF_PPT; ++i) {
-        const int c = tid + 256 * i < PF_PIECES ? tid + 256 * i : 0;
-        int key = blk + c / (D / 8);
-        key = key < kmax ? key : kmax;
-        int rel = key - walk_start;
-        int w = (rel >= page ? 1 : 0) + (rel >= 2 * page ? 1 : 0);
-        Wh.kpg[i] = bt[walk_idx + w];
-        Wh.koff[i] = rel - w * page;
-        key = blk + (c & 3) * 8;
-        key = key < (kmax & ~7) ? key : (kmax & ~7);
-        rel = key - walk_start;
-        w = (rel >= page ? 1 : 0) + (rel >= 2 * page ? 1 : 0);
-        Wh.vpg[i] = bt[walk_idx + w];
-        Wh.voff[i] = rel - w * page;
+        const int c = tid + PF_COPIERS * i;
+        int key;
+        if (c < PF_PIECES / 2) {                       // keys: dims 16 j .. 16 j + 15 of key c / (D / 16)
+          key = blk + c / (D / 16);
+          key = key < kmax ? key : kmax;
+        } else {                                       // values: keys 16 g .. 16 g + 15 of one dim, g = c % 2
+          key = blk + (c & 1) * 16;
+          key = key < (kmax & ~15) ? key : (kmax & ~15);
+        }
+        const int rel = key - walk_start;
+        const int w = (rel >= page ? 1 : 0) + (rel >= 2 * page ? 1 : 0);
+        Wh.pg[i] = bt[walk_idx + w];
+        Wh.off[i] = rel - w * page;
       }
     };
     auto fetch = [&](Pieces& P, const Where& Wh) {
+      if (!copier) return;
 #pragma unroll
       for (int i = 0; i < PF_PPT; ++i) {
-        const int c = tid + 256 * i < PF_PIECES ? tid + 256 * i : 0;
-        P.k[i] = *reinterpret_cast<const uint4*>(
-            k_cache + (((size_t)Wh.kpg[i] * Hkv + kvh) * page + Wh.koff[i]) * D + (c % (D / 8)) * 8);
-        P.v[i] = *reinterpret_cast<const uint4*>(
-            v_cache + (((size_t)Wh.vpg[i] * Hkv + kvh) * D + (c >> 2)) * page + Wh.voff[i]);
+        const int c = tid + PF_COPIERS * i;
+        const bf16* src = nullptr;
+        if (c < PF_PIECES / 2)
+          src = k_cache + (((size_t)Wh.pg[i] * Hkv + kvh) * page + Wh.off[i]) * D + (c % (D / 16)) * 16;
+        else if (c < PF_PIECES)
+          src = v_cache + (((size_t)Wh.pg[i] * Hkv + kvh) * D + ((c - PF_PIECES / 2) >> 1)) * page + Wh.off[i];
+        if (src) {
+          P.lo[i] = *reinterpret_cast<const uint4*>(src);
+          P.hi[i] = *reinterpret_cast<const uint4*>(src + 8);
+        }
       }
     };
     auto stash = [&](Pieces& P, int buf, int blk) {
+      if (!copier) return;
       unsigned char* base = pf_lds + buf * PF_BUF;
 #pragma unroll
       for (int i = 0; i < PF_PPT; ++i) {
-        const int c = tid + 256 * i;
-        if (c >= PF_PIECES) continue;
-        *reinterpret_cast<uint4*>(base + (c / (D / 8)) * PF_KROW + (c % (D / 8)) * 16) = P.k[i];
-        uint4 v = P.v[i];
-        const int key0 = blk + (c & 3) * 8;
-        if (key0 + 7 > kmax) {
-          // slots after the row's last key may be stale: zero them (0 * NaN must not reach the sum)
-          uint32_t* w = reinterpret_cast<uint32_t*>(&v);
+        const int c = tid + PF_COPIERS * i;
+        if (c < PF_PIECES / 2) {
+          unsigned char* at = base + (c / (D / 16)) * PF_KROW + (c % (D / 16)) * 32;
+          *reinterpret_cast<uint4*>(at) = P.lo[i];
+          *reinterpret_cast<uint4*>(at + 16) = P.hi[i];
+        } else if (c < PF_PIECES) {
+          const int cv = c - PF_PIECES / 2;
+          uint32_t w[8] = {P.lo[i].x, P.lo[i].y, P.lo[i].z, P.lo[i].w, P.hi[i].x, P.hi[i].y, P.hi[i].z, P.hi[i].w};
+          const int key0 = blk + (cv & 1) * 16;
+          if (key0 + 15 > kmax) {
+            // slots after the row's last key may be stale: zero them (0 * NaN must not reach the sum)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (key0 + 2 * e > kmax) w[e] &= 0xFFFF0000u;
-            if (key0 + 2 * e + 1 > kmax) w[e] &= 0x0000FFFFu;
+            for (int e = 0; e < 8; ++e) {
+              if (key0 + 2 * e > kmax) w[e] &= 0xFFFF0000u;
+              if (key0 + 2 * e + 1 > kmax) w[e] &= 0x0000FFFFu;
+            }
           }
+          // within a row the keys stand in the order the second product wants them: keys 4 g .. 4 g + 3 and
+          // 16 + 4 g .. 16 + 4 g + 3 side by side, so that a lane's eight values are one 16-byte read
+          unsigned char* at = base + PF_KBYTES + (cv >> 1) * PF_VROW + (cv & 1) * 8;
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) *reinterpret_cast<uint2*>(at + 16 * g4) = make_uint2(w[2 * g4], w[2 * g4 + 1]);
         }
-        *reinterpret_cast<uint4*>(base + PF_KBYTES + (c >> 2) * PF_VROW + (c & 3) * 16) = v;
       }
     };
 
@@ -180,9 +207,8 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
         }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
-        const unsigned char* vr = Vb + (dt * 16 + col) * PF_VROW + 8 * kb;
-        va[dt].h[0] = *reinterpret_cast<const uint2*>(vr);
-        va[dt].h[1] = *reinterpret_cast<const uint2*>(vr + 32);
+        const unsigned char* vr = Vb + (dt * 16 + col) * PF_VROW + 16 * kb;
+        va[dt].q = *reinterpret_cast<const uint4*>(vr);
       }
       f32x4 S[PF_NT][2];
       bool whole = true;      // every query of every tile sees every key of the block (uniform over the wave)
@@ -263,25 +289,37 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
           O[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt].v, pb[j].v, O[j][dt], 0, 0, 0);
     };
 
-    // ---- the blocks, two buffers: block i is computed while block i + 1 travels and the pages of block
-    // i + 2 are looked up; one barrier a block
-    Where wh_next;
-    Pieces pc;
-    lookup(wh_next, blk0);
-    fetch(pc, wh_next);
-    lookup(wh_next, blk0 + BLOCK_KEYS);
+    // ---- the blocks, two LDS buffers and two sets of registers: while block i is computed, block i + 1
+    // sits in registers (asked for an iteration ago, stored to the LDS after the computing), block i + 2 is
+    // on its way from memory and the pages of block i + 3 are looked up.  One barrier a block.
+    Where wh;
+    Pieces pa, pb;
+    lookup(wh, blk0);
+    fetch(pa, wh);                                     // block 0
+    lookup(wh, blk0 + BLOCK_KEYS);
+    fetch(pb, wh);                                     // block 1 (clamped into the row if there is none)
+    lookup(wh, blk0 + 2 * BLOCK_KEYS);
     __syncthreads();                                   // the previous stretch is done with the buffers
-    stash(pc, 0, blk0);
+    stash(pa, 0, blk0);
     __syncthreads();
-    int buf = 0;
-    for (int blk = blk0; blk <= kmax; blk += BLOCK_KEYS, buf ^= 1) {
-      const bool more = blk + BLOCK_KEYS <= kmax;      // uniform over the workgroup
-      if (more) {
-        fetch(pc, wh_next);
-        lookup(wh_next, blk + 2 * BLOCK_KEYS);
+    auto mine = [&](int blk) { return blk <= wave_kmax && blk + BLOCK_KEYS > wave_kmin; };
+    for (int blk = blk0; blk <= kmax; blk += 2 * BLOCK_KEYS) {      // every condition is uniform over the workgroup
+      // block blk from buffer 0; pb holds block blk + 32; pa is free for block blk + 64
+      if (blk + 2 * BLOCK_KEYS <= kmax) {
+        fetch(pa, wh);
+        lookup(wh, blk + 3 * BLOCK_KEYS);
       }
-      if (blk <= wave_kmax && blk + BLOCK_KEYS > wave_kmin) compute(buf, blk);
-      if (more) stash(pc, buf ^ 1, blk + BLOCK_KEYS);
+      if (mine(blk)) compute(0, blk);
+      if (blk + BLOCK_KEYS > kmax) break;              // (no barrier needed: nothing reads the LDS after this)
+      stash(pb, 1, blk + BLOCK_KEYS);
+      __syncthreads();
+      // block blk + 32 from buffer 1; pa holds block blk + 64; pb is free for block blk + 96
+      if (blk + 3 * BLOCK_KEYS <= kmax) {
+        fetch(pb, wh);
+        lookup(wh, blk + 4 * BLOCK_KEYS);
+      }
+      if (mine(blk + BLOCK_KEYS)) compute(1, blk + BLOCK_KEYS);
+      if (blk + 2 * BLOCK_KEYS <= kmax) stash(pa, 0, blk + 2 * BLOCK_KEYS);
       __syncthreads();
     }
 
@@ -321,9 +359,10 @@ MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k
   int hpw = PF_NT;                       // heads of a kv group per wave: the largest power of two <= min(G, PF_NT)
   while (hpw > G) hpw >>= 1;
   const int head_waves = (G + hpw - 1) / hpw;
-  const int waves_h = head_waves >= 3 ? 4 : head_waves;       // waves side by side over the heads: 1, 2 or 4
+  int waves_h = 1;                       // waves side by side over the heads: a power of two up to PF_WAVES
+  while (waves_h < head_waves && waves_h < PF_WAVES) waves_h <<= 1;
   const int head_chunks = (G + hpw * waves_h - 1) / (hpw * waves_h);
-  const int stretch = (4 / waves_h) * (PF_NT / hpw) * 16;      // queries a workgroup serves at a time
+  const int stretch = (PF_WAVES / waves_h) * (PF_NT / hpw) * 16;      // queries a workgroup serves at a time
   const long stretches = (max_row_tokens + stretch - 1) / stretch;
   const long gx = (stretches + 1) / 2;                        // a workgroup takes a late stretch and an early one
   if (rows > 65535 || (long)Hkv * head_chunks > 65535) MIE_FAIL("prefill_attention: grid too large (%d rows)", rows);
@@ -339,7 +378,7 @@ MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k
       lds_allowed[dev] = true;
     }
   }
-  dim3 grid((unsigned)gx, rows, Hkv * head_chunks), block(256);
+  dim3 grid((unsigned)gx, rows, Hkv * head_chunks), block(PF_THREADS);
   hipLaunchKernelGGL(prefill_attention_kernel, grid, block, lds_bytes, stream, (const bf16*)q, q_stride,
                      (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, block_tables, max_blocks, row_start,
                      row_position, first_row, Hq, Hkv, hpw, waves_h, page, scale * 1.4426950408889634f, window);
