@@ -187,6 +187,30 @@ def test_generate_b_gpu(tiny_models, dtype, graphs):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_a_step_ahead_gpu(tiny_models, dtype):
+    """On the device the next step's rows take their tokens from the sampling kernel's output buffer (captured
+    graphs included); stop tokens are seen a step late.  Same tokens as with every step read before the next."""
+    m = tiny_models["B"]
+    prompts = prompts_for(m, [3, 25, 9, 40, 14, 1], seed=12)
+    sp_free = SamplingParams(max_tokens=30, ignore_eos=True)
+    free_run = engine(m, "cuda", dtype, num_blocks=40, max_num_seqs=6, run_ahead=False).generate(prompts, sp_free)
+    stop = free_run[2].output_ids[5]
+    params = [SamplingParams(max_tokens=30 - 3 * i, temperature=0.7 if i % 2 else 0.0, seed=50 + i) for i in range(6)]
+    results = {}
+    for ahead in (False, True):
+        eng = engine(m, "cuda", dtype, num_blocks=40, max_num_seqs=6, max_num_batched_tokens=24, run_ahead=ahead,
+                     graph_batch_sizes=(1, 2, 4, 8))
+        eng.eos_token_id = stop
+        results[ahead] = [o.output_ids for o in eng.generate(prompts, params)]
+        eng.cache.check()
+        assert not eng.cache.live and not eng.has_work()
+        assert eng.num_graph_steps > 5
+    assert any(ids and ids[-1] == stop and len(ids) < 12 for ids in results[False]), "no request ended by the stop token"
+    assert results[True] == results[False]
+
+
+@pytest.mark.gpu
 def test_graph_steps_equal_eager_steps(tiny_models):
     """Captured decode steps replayed many times, with eager work in between, give the eager tokens."""
     m = tiny_models["C"]
