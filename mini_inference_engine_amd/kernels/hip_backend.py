@@ -51,6 +51,7 @@ class HipBackend(KernelBackend):
             raise RuntimeError("no GPU visible to torch: the engine needs an MI355X (gfx950)")
         self._libs = {}
         self.true_fp32 = act_dtype == torch.float32
+        self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
 
     # ------------------------------------------------------------ plumbing
     def lib(self, module: str, defines: tuple = ()):
@@ -114,7 +115,8 @@ class HipBackend(KernelBackend):
             fn.restype = c_int
 
     def _stream(self) -> c_void_p:
-        return c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        # the handle alone: building torch's Stream object costs several microseconds a launch
+        return c_void_p(torch._C._cuda_getCurrentRawStream(self._device_index))
 
     def _on_device(self, *tensors) -> None:
         for t in tensors:
