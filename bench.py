@@ -34,7 +34,7 @@ REFERENCE_B8_TOKENS_PER_S = 8 / 10.02e-3
 
 
 def tinyllama_config(layers: int | None = None):
-    """Layer sizes of BASELINE.json configs[2]."""
+    """TinyLlama-1.1B layer sizes, the configuration the benchmark is quoted on."""
     from mini_inference_engine_amd.config import LlamaConfig
     return LlamaConfig(vocab_size=32000, hidden_size=2048, intermediate_size=5632,
                        num_hidden_layers=layers or 22, num_attention_heads=32, num_key_value_heads=4, head_dim=64,

@@ -15,7 +15,7 @@ import sys
 import tempfile
 
 SHAPES = {
-    # BASELINE configurations: tiny A and B of the tests, and the benchmark's layer sizes
+    # the two tiny configurations of the tests, the benchmark's layer sizes, and two larger models' sizes
     "tiny-a": dict(vocab_size=256, hidden_size=64, intermediate_size=176, num_hidden_layers=2, num_attention_heads=4,
                    num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-5, rope_theta=10000.0,
                    max_position_embeddings=128, tie_word_embeddings=False),
