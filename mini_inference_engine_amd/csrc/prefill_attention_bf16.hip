@@ -41,22 +41,44 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
                          const int* __restrict__ row_position, int first_row, int Hq, int Hkv, int hpw,
                          int waves_h, int page, float scale_log2, int window) {
   extern __shared__ __align__(16) unsigned char pf_lds[];
-  const int row = first_row + blockIdx.y;
+  // Which (stretch pair, row, kv head) this workgroup takes.  Workgroups go to the eight XCDs in turn, in
+  // launch order with x fastest, and every XCD has an L2 of its own: all workgroups of one kv head read
+  // the same keys and values, so they are placed on one XCD (or on 8 / Z of them when there are fewer
+  // than eight z indices), and a block of keys is fetched into one L2 instead of all eight.
+  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  {
+    const unsigned X = gridDim.x, Y = gridDim.y, Z = gridDim.z;
+    const unsigned w = blockIdx.x + X * (blockIdx.y + Y * blockIdx.z), total = X * Y * Z;
+    if (total % 8 == 0 && (Z % 8 == 0 || 8 % Z == 0)) {       // uniform over the grid
+      unsigned r;
+      if (Z % 8 == 0) {
+        bz = (int)(w % 8 + 8 * ((w / 8) % (Z / 8)));
+        r = w / Z;
+      } else {
+        const unsigned c = w % 8;
+        bz = (int)(c % Z);
+        r = (w / 8) * (8 / Z) + c / Z;
+      }
+      bx = (int)(r % X);
+      by = (int)(r / X);
+    }
+  }
+  const int row = first_row + by;
   const int G = Hq / Hkv;
   const int qpw = PF_NT / hpw, waves_q = PF_WAVES / waves_h, QT = waves_q * qpw;
   const int head_chunks = (G + hpw * waves_h - 1) / (hpw * waves_h);
-  const int kvh = blockIdx.z / head_chunks, hc = blockIdx.z - kvh * head_chunks;
+  const int kvh = bz / head_chunks, hc = bz - kvh * head_chunks;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, kb = lane >> 4;
   const int t0 = row_start[row], q_len = row_start[row + 1] - t0, p0 = row_position[row];
   const int NS = (q_len + 16 * QT - 1) / (16 * QT);          // stretches of this row
-  if ((int)blockIdx.x >= (NS + 1) / 2) return;               // the whole workgroup, before any barrier
+  if (bx >= (NS + 1) / 2) return;               // the whole workgroup, before any barrier
   const int wh = wave % waves_h, wq = wave / waves_h;
   const int* bt = block_tables + (size_t)row * max_blocks;
 
   for (int pass = 0; pass < 2; ++pass) {
-    const int s = pass == 0 ? NS - 1 - (int)blockIdx.x : (int)blockIdx.x;
-    if (pass == 1 && s >= NS - 1 - (int)blockIdx.x) break;   // the middle stretch of an odd number has no partner
+    const int s = pass == 0 ? NS - 1 - bx : bx;
+    if (pass == 1 && s >= NS - 1 - bx) break;   // the middle stretch of an odd number has no partner
 
     // ---- this wave's tiles
     bool tile_ok[PF_NT], q_ok[PF_NT];
