@@ -242,32 +242,40 @@ merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ 
   float acc[DL];
 #pragma unroll
   for (int i = 0; i < DL; ++i) acc[i] = 0.f;
+  // Sixteen splits' partial outputs at a time.  The first sixteen are asked for before their weights are
+  // known, so that the kernel waits for memory once and not twice; every load is unconditional, from an
+  // address clamped into the operand (what is read for a split or a dim that does not exist is not used).
+  float part[16][DL];
+  auto ask = [&](int first) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+#pragma unroll
+      for (int i = 0; i < DL; ++i) {
+        const int d = lane + 64 * i, sp = first + j;
+        part[j][i] = op[(size_t)(sp < num_splits ? sp : num_splits - 1) * D + (d < D ? d : 0)];
+      }
+  };
+  ask(0);
   float W = 0.f;
   float M = -INFINITY;                       // the maximum over all splits first (64 a round)
   for (int s0 = 0; s0 < num_splits; s0 += 64) {
-    const float v = s0 + lane < num_splits ? lse[s0 + lane] : -INFINITY;
-    M = fmaxf(M, wave_max(v));
+    const float v = lse[s0 + lane < num_splits ? s0 + lane : 0];
+    M = fmaxf(M, wave_max(s0 + lane < num_splits ? v : -INFINITY));
   }
   for (int s0 = 0; s0 < num_splits; s0 += 64) {
-    const float v = s0 + lane < num_splits ? lse[s0 + lane] : -INFINITY;
+    const float vv = lse[s0 + lane < num_splits ? s0 + lane : 0];
+    const float v = s0 + lane < num_splits ? vv : -INFINITY;
     const float w = v == -INFINITY ? 0.f : exp2f(v - M);
     W += wave_sum(w);
     const int n = num_splits - s0 < 64 ? num_splits - s0 : 64;
     for (int c = 0; c < n; c += 16) {
-      float part[16][DL];
-#pragma unroll
-      for (int j = 0; j < 16; ++j)
-#pragma unroll
-        for (int i = 0; i < DL; ++i) {
-          const int d = lane + 64 * i;
-          part[j][i] = (c + j < n && d < D) ? op[(size_t)(s0 + c + j) * D + d] : 0.f;
-        }
+      if (s0 + c > 0) ask(s0 + c);
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const float wj = __shfl(w, (c + j) & 63, 64);
 #pragma unroll
         for (int i = 0; i < DL; ++i)
-          if (c + j < n && wj != 0.f) acc[i] += wj * part[j][i];    // a split without keys holds no data
+          if (c + j < n && wj != 0.f && lane + 64 * i < D) acc[i] += wj * part[j][i];    // a split without keys holds no data
       }
     }
   }
