@@ -79,6 +79,17 @@ add_rmsnorm_kernel(const TX* __restrict__ x, float* __restrict__ stream, const T
 #define NORM_FAST_THREADS 256
 #define NORM_FAST_VEC 8      // float4 groups per thread: widths up to 8192
 
+// four elements as they lie in memory, and as numbers
+template <typename T> struct Raw4;
+template <> struct Raw4<float> { float4 v; };
+template <> struct Raw4<bf16> { uint2 v; };
+__device__ __forceinline__ Raw4<float> load_raw(const float* p) { return Raw4<float>{*reinterpret_cast<const float4*>(p)}; }
+__device__ __forceinline__ Raw4<bf16> load_raw(const bf16* p) { return Raw4<bf16>{*reinterpret_cast<const uint2*>(p)}; }
+__device__ __forceinline__ float4 to_float4(const Raw4<float>& r) { return r.v; }
+__device__ __forceinline__ float4 to_float4(const Raw4<bf16>& r) {
+  return make_float4(__uint_as_float(r.v.x << 16), __uint_as_float(r.v.x & 0xFFFF0000u), __uint_as_float(r.v.y << 16),
+                     __uint_as_float(r.v.y & 0xFFFF0000u));
+}
 template <typename T> __device__ __forceinline__ float4 load4(const T* p);
 template <> __device__ __forceinline__ float4 load4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
 template <> __device__ __forceinline__ float4 load4<bf16>(const bf16* p) {
@@ -103,20 +114,30 @@ add_rmsnorm_fast_kernel(const TX* __restrict__ x, float* __restrict__ stream, co
   const int row = rows ? rows[out_row] : out_row;
   float* sr = stream + (size_t)row * width;
   const TX* xr = x ? x + (size_t)row * width : nullptr;
-  float4 r[NORM_FAST_VEC], w[NORM_FAST_VEC];
+  // first every load, as it comes from memory (a conversion or an add where a value is loaded would make
+  // the compiler wait for it there, one memory latency per group of four instead of one in all)
+  Raw4<float> r_raw[NORM_FAST_VEC];
+  Raw4<TW> w_raw[NORM_FAST_VEC];
+  Raw4<TX> a_raw[NORM_FAST_VEC];
 #pragma unroll
   for (int k = 0; k < NORM_FAST_VEC; ++k) {
     const int i = (threadIdx.x + k * NORM_FAST_THREADS) * 4;
-    r[k] = make_float4(0.f, 0.f, 0.f, 0.f);
-    w[k] = r[k];
+    r_raw[k] = Raw4<float>{};
+    w_raw[k] = Raw4<TW>{};
+    a_raw[k] = Raw4<TX>{};
     if (i < width) {
-      r[k] = load4(sr + i);
-      w[k] = load4(weight + i);
-      if (xr) {
-        const float4 a = load4(xr + i);
-        r[k].x += a.x; r[k].y += a.y; r[k].z += a.z; r[k].w += a.w;
-      }
+      r_raw[k] = load_raw(sr + i);
+      w_raw[k] = load_raw(weight + i);
+      if (xr) a_raw[k] = load_raw(xr + i);
     }
+  }
+  float4 r[NORM_FAST_VEC], w[NORM_FAST_VEC];
+#pragma unroll
+  for (int k = 0; k < NORM_FAST_VEC; ++k) {
+    r[k] = to_float4(r_raw[k]);
+    w[k] = to_float4(w_raw[k]);
+    const float4 a = to_float4(a_raw[k]);          // zeros where nothing was loaded
+    r[k].x += a.x; r[k].y += a.y; r[k].z += a.z; r[k].w += a.w;
   }
   float ss = 0.f;
 #pragma unroll
