@@ -93,6 +93,13 @@ class CacheManager:
         """All groups or none (inference_engine/block_manager.py:32-40)."""
         if rc.closed:
             raise CacheAccountingError(f"request {rc.request_id!r} is closed")
+        # most calls are a decoding request whose next token still fits its last page: nothing to do
+        end = num_computed + n
+        for t in rc.tables:
+            if len(t) * self.page_size < end:
+                break
+        else:
+            return True
         if not self.can_reserve(rc, num_computed, n, watermark):
             return False
         for g, k in enumerate(self.pages_needed(rc, num_computed, n)):
