@@ -321,3 +321,63 @@ MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_
   return 0;
 }
 
+
+// ---- the same for callers that cannot allocate (decode_attention_static.hpp)
+#include "decode_attention_static.hpp"
+#include <mutex>
+
+// Partial results of a split context: the library's own device memory, one copy on every GPU.
+// In host code this name is only a stand-in for the symbol; the device address comes from
+// hipGetSymbolAddress, per device, and only that address is ever handed to a kernel.
+static __device__ __align__(256) float scratch[MIE_DECODE_STATIC_SCRATCH_BYTES / sizeof(float)];
+
+constexpr int MAX_DEVICES = 64;
+static float* g_scratch_of_device[MAX_DEVICES];
+static std::mutex g_scratch_lock;
+
+static int scratch_for_current_device(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) MIE_FAIL("decode_attention_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= MAX_DEVICES) MIE_FAIL("decode_attention_static: device %d (at most %d devices)", dev, MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_of_device[dev]) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      MIE_FAIL("decode_attention_static: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_of_device[dev] = p;
+  }
+  *ptr = g_scratch_of_device[dev];
+  return 0;
+}
+
+MIE_EXPORT int mie_decode_attention_static_setup(void) {
+  float* p;
+  return scratch_for_current_device(&p);
+}
+
+MIE_EXPORT long mie_decode_attention_static_capacity(void) { return (long)MIE_DECODE_STATIC_SCRATCH_BYTES; }
+
+MIE_EXPORT int mie_decode_attention_static(const void* q, long q_stride, const void* k_cache, const void* v_cache,
+                                           void* out, const int* block_tables, int max_blocks, const int* positions,
+                                           int rows, int Hq, int Hkv, int head_dim, int page, float scale, int window,
+                                           int partition, int num_splits, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (num_splits <= 1)      // no partial results: the plain entry point allocates nothing either
+    return mie_decode_attention(q, q_stride, k_cache, v_cache, out, nullptr, nullptr, block_tables, max_blocks,
+                                positions, rows, Hq, Hkv, head_dim, page, scale, window, partition, num_splits, stream);
+  if (Hq <= 0 || head_dim != D) MIE_FAIL("decode_attention_static: built for head_dim %d, called with %d (%d heads)", D, head_dim, Hq);
+  const size_t entries = (size_t)rows * (size_t)Hq * (size_t)num_splits;
+  const size_t need = entries * (D + 1) * sizeof(float);
+  if (need > MIE_DECODE_STATIC_SCRATCH_BYTES)
+    MIE_FAIL("decode_attention_static: %d rows x %d heads x %d splits x head_dim %d need %zu bytes for partial results; "
+             "the library holds %u (fewer splits, or the entry point that takes buffers)",
+             rows, Hq, num_splits, D, need, (unsigned)MIE_DECODE_STATIC_SCRATCH_BYTES);
+  float* base = nullptr;
+  if (scratch_for_current_device(&base)) return -1;
+  float* o_part = base;                       // [rows, Hq, splits, D]
+  float* lse_part = base + entries * D;       // [rows, Hq, splits]
+  return mie_decode_attention(q, q_stride, k_cache, v_cache, out, o_part, lse_part, block_tables, max_blocks, positions,
+                              rows, Hq, Hkv, head_dim, page, scale, window, partition, num_splits, stream);
+}
