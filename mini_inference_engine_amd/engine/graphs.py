@@ -16,10 +16,10 @@ import torch
 
 
 class DecodeGraphs:
-    def __init__(self, runner, cfg, verbose: bool = True):
+    def __init__(self, runner, batch_sizes, verbose: bool = True):
         self.runner = runner
-        self.sizes = sorted(b for b in set(cfg.graph_batch_sizes) if b <= cfg.max_num_seqs
-                            and b <= cfg.max_num_batched_tokens)
+        arena = runner.arena
+        self.sizes = sorted(b for b in set(batch_sizes) if 0 < b <= arena.max_rows and b <= arena.max_tokens)
         self.graphs = {}
         self.static_context = runner.max_model_len
         if not self.sizes:

@@ -73,10 +73,9 @@ class LLMEngine:
         if load_tokenizer and isinstance(model, str):
             from transformers import AutoTokenizer      # text in and out only; never on the token path
             self.tokenizer = AutoTokenizer.from_pretrained(model)
-        self.graphs = None
         if cfg.use_hip_graphs and self.runner.device.type == "cuda":
-            from .graphs import DecodeGraphs
-            self.graphs = DecodeGraphs(self.runner, cfg, verbose=verbose)
+            self.runner.capture_decode_graphs(cfg.graph_batch_sizes, verbose=verbose)
+        self.graphs = self.runner.graphs
         self.num_steps = 0
         self.num_graph_steps = 0
         self._num_requests = 0
@@ -153,13 +152,9 @@ class LLMEngine:
             if last:
                 sample_seqs.append(seq)
 
-        pure_decode = all(n == 1 for _, n in batch)
-        if pure_decode and self.graphs is not None and self.graphs.fits(len(rows)):
-            logits = self.graphs.run(rows)
-            self.num_graph_steps += 1
-        else:
-            logits = self.runner.forward_step(rows)
+        logits = self.runner.forward_step(rows)       # a captured graph when every row is a single token
         self.num_steps += 1
+        self.num_graph_steps += self.runner.last_step_captured
 
         chosen = None
         if sample_seqs:

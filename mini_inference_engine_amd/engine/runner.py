@@ -82,6 +82,8 @@ class ModelRunner:
         # The tokens the last step chose, at a fixed address: the next step's rows may take their token
         # from here on the device (StepRow.taken_from) before the host has seen it.
         self.chosen_tokens = torch.zeros(max(1, max_rows), dtype=torch.int32, device=self.device)
+        self.graphs = None                  # captured decode steps, once capture_decode_graphs was called
+        self.last_step_captured = False
 
     # ------------------------------------------------------------------ steps
     def build(self, rows: list[StepRow], **kw):
@@ -95,10 +97,21 @@ class ModelRunner:
         step.earlier_tokens = self.chosen_tokens
         return step
 
+    def capture_decode_graphs(self, batch_sizes, verbose: bool = False) -> None:
+        """Capture the forward of a step of single-token rows once per batch size; ``forward_step``
+        then replays the smallest captured size that holds such a step instead of launching kernel by
+        kernel (inference_engine/engine.py:76-120)."""
+        from .graphs import DecodeGraphs
+        self.graphs = DecodeGraphs(self, batch_sizes, verbose=verbose)
+
     @torch.inference_mode()
     def forward_step(self, rows: list[StepRow]) -> torch.Tensor | None:
         """Logits [sum of wants, vocab] float32, ordered by row then by ``want``.
         Pages for the rows' tokens must have been reserved."""
+        self.last_step_captured = False
+        if self.graphs is not None and self.graphs.fits(len(rows)) and all(len(r.tokens) == 1 for r in rows):
+            self.last_step_captured = True
+            return self.graphs.run(rows)
         step = self.build(rows)
         return self.model.forward(step)
 

@@ -248,7 +248,11 @@ class HipBackend(KernelBackend):
             self._skinny(x, w, self.EPI_BF16 if out_dtype == torch.bfloat16 else self.EPI_F32, out, N)
             return out
         if not self.true_fp32 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
-            # library matrix product, 32-bit accumulation, as the reference's F.linear
+            # library matrix product, 32-bit accumulation, as the reference's F.linear.  What goes into the
+            # float32 stream or out as logits leaves the product in float32: the sums are not rounded to
+            # bfloat16 on their way there, whatever the number of rows.
+            if bias is None and (sink is not None or out_dtype == torch.float32):
+                return torch.mm(x, w.t(), out_dtype=torch.float32)
             y = torch.nn.functional.linear(x, w, None if bias is None else bias.to(torch.bfloat16))
             return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
         return self._gemm(x, w, bias, out_dtype)

@@ -28,7 +28,10 @@ def _parser():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time; sizes the page pool")
+                    help="most tokens live requests hold at any time, each request's count rounded up to a "
+                         "multiple of 64 (or of the page size if that is larger); sizes the page pool")
+    ap.add_argument("--hip-graphs", action="store_true",
+                    help="run steps of single-token entries through captured graphs, as generation does")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--device", default="cuda")
     return ap
@@ -89,6 +92,8 @@ def main(argv=None) -> int:
     pages = -(-args.max_tokens // page) + 1          # + the scratch page
     runner = ModelRunner(args.model, dtype=args.dtype, device=args.device, page_size=page, num_pages=pages,
                          max_step_tokens=max(64, args.max_tokens), max_rows=64)
+    if args.hip_graphs:
+        runner.capture_decode_graphs((1, 2, 4, 8))
 
     def say(msg):
         print(msg, flush=True)

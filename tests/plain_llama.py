@@ -1,7 +1,7 @@
 """A plain, slow Llama: whole sequences, no cache, no batching, one function per part.
 
-Written from the reference's formulas (each function cites file:line of
-/root/reference); it shares no code with the engine.  Weights come as the
+Written from the reference's formulas (each function cites file:line of the
+reference's tree, inference_engine/...); it shares no code with the engine.  Weights come as the
 name -> tensor dict of a checkpoint.  Everything runs in ``dtype`` (float64 by
 default, so that the oracle's own rounding is far below what it judges), except
 the rotary angle table, which the reference computes in float32 by formula and
@@ -49,8 +49,8 @@ def causal_attention(q, k, v, scale, window=None):
     ke = k.repeat_interleave(g, dim=1)
     ve = v.repeat_interleave(g, dim=1)
     s = torch.einsum("ihd,jhd->hij", q, ke) * scale
-    i = torch.arange(n)[:, None]
-    j = torch.arange(n)[None, :]
+    i = torch.arange(n, device=q.device)[:, None]
+    j = torch.arange(n, device=q.device)[None, :]
     seen = j <= i
     if window is not None:
         seen &= j > i - window
@@ -93,13 +93,15 @@ def forward(cfg: dict, weights: dict, token_ids, dtype=torch.float64, position_o
     """Logits [n, vocab] of one whole sequence (inference_engine/model.py:161-185).
     Residual wiring: stream = embed; stream += attention(norm(stream)); stream +=
     mlp(norm(stream)); logits = lm_head(norm(stream)).  ``position_offset`` shifts all
-    positions (for the invariance test; the engine always starts at 0)."""
+    positions (for the invariance test; the engine always starts at 0).  Runs where the
+    weights are (a model of real width is judged on the GPU, with torch's float64)."""
     cfg = normalise_config(cfg)
     w = {k: v.to(dtype) for k, v in weights.items()}
-    ids = torch.as_tensor(token_ids, dtype=torch.long)
+    device = w["model.embed_tokens.weight"].device
+    ids = torch.as_tensor(token_ids, dtype=torch.long, device=device)
     n = ids.shape[0]
     cos, sin = rope_table(cfg["rope_theta"], cfg["head_dim"], position_offset + n)
-    cos, sin = cos[position_offset:].to(dtype), sin[position_offset:].to(dtype)
+    cos, sin = cos[position_offset:].to(device, dtype), sin[position_offset:].to(device, dtype)
     eps = cfg["rms_norm_eps"]
     stream = w["model.embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):

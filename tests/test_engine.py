@@ -211,6 +211,26 @@ def test_running_a_step_ahead_gpu(tiny_models, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_requests_at_once_gpu(tiny_models, dtype):
+    """48 requests together: decode steps of 33 to 48 rows (beyond the few-row kernels), captured at batch
+    sizes 48 and 64, tokens handed from step to step on the device, greedy and sampled rows side by side."""
+    m = tiny_models["B"]
+    lengths = [1 + (7 * i) % 40 for i in range(48)]
+    prompts = prompts_for(m, lengths, seed=21)
+    params = [SamplingParams(max_tokens=6, temperature=0.0 if i % 3 else 0.9, ignore_eos=True, seed=300 + i)
+              for i in range(48)]
+    eng = engine(m, "cuda", dtype, num_blocks=48 * 4 + 1, max_num_seqs=64, max_num_batched_tokens=512,
+                 graph_batch_sizes=(48, 64))
+    outs = eng.generate(prompts, params)
+    assert eng.num_graph_steps >= 4, "the steps of 48 single-token rows did not go through the captured graphs"
+    check_outputs(m, prompts, outs, params, 1e-5 if dtype == "float32" else 2e-2,
+                  "weights" if dtype == "float32" else "weights_bf16")
+    eng.cache.check()
+    assert not eng.cache.live
+
+
+@pytest.mark.gpu
 def test_graph_steps_equal_eager_steps(tiny_models):
     """Captured decode steps replayed many times, with eager work in between, give the eager tokens."""
     m = tiny_models["C"]

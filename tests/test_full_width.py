@@ -1,0 +1,162 @@
+"""The whole model at the layer sizes of TinyLlama-1.1B (width 2048, 32 query heads on 4 kv heads of 64,
+feed-forward 5632, vocabulary 32000) with random weights, against the plain implementation run in
+float64 on the GPU.  The reference's only generation test runs these sizes (tests/test_correctness.py:41-101
+there); here it is the logits that are compared, in float32 and in bfloat16:
+
+  * one whole prompt of 300 tokens;
+  * most of it in one step and the last 32 tokens one by one through the captured decode graph;
+  * steps of 40 and of 64 single-token rows, launched kernel by kernel and through captured graphs
+    (the few-row kernels end at 32 rows; buckets 48 and 64).
+
+The number of layers is LAYERS (the configuration has 22): what a layer does to the stream is the same in
+every layer, and the depth the engine's other tests reach is 3.
+"""
+import pytest
+import torch
+
+import plain_llama
+
+pytestmark = pytest.mark.gpu
+
+LAYERS = 22
+CFG = dict(architectures=["LlamaForCausalLM"], vocab_size=32000, hidden_size=2048, intermediate_size=5632,
+           num_hidden_layers=LAYERS, num_attention_heads=32, num_key_value_heads=4, head_dim=64,
+           rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=2048, tie_word_embeddings=False,
+           eos_token_id=2)
+F32_TOL = 2e-5      # of the request's logit scale
+BF16_TOL = 2e-2
+PROMPT = 300
+TAIL = 32
+
+
+@pytest.fixture(scope="module")
+def model():
+    from mini_inference_engine_amd.config import LlamaConfig
+    from mini_inference_engine_amd.weights import random_tensors
+    config = LlamaConfig.from_dict(CFG)
+    w32 = random_tensors(config, 2, torch.float32, device="cuda")
+    return {"config": config,
+            "float32": w32,
+            "bfloat16": {k: v.to(torch.bfloat16) for k, v in w32.items()}}
+
+
+def make_runner(model, dtype, pages, max_rows=64, max_step_tokens=512):
+    from mini_inference_engine_amd.engine.runner import ModelRunner
+    r = ModelRunner(model["config"], weights=model[dtype], dtype=dtype, device="cuda", num_pages=pages,
+                    max_rows=max_rows, max_step_tokens=max_step_tokens)
+    assert r.ops.name == "hip-gfx950"
+    return r
+
+
+def plain_logits(model, dtype, tokens):
+    key = dtype + " widened"
+    if key not in model:
+        model[key] = {k: v.double() for k, v in model[dtype].items()}
+    return plain_llama.forward(CFG, model[key], tokens, torch.float64)
+
+
+def worst_error(got, expect, tol, what, scale=None):
+    """got [n, vocab] float32 against expect [n, vocab] float64, in units of ``scale`` (the request's
+    largest logit; by default the largest of ``expect``)."""
+    scale = scale or float(expect.abs().max())
+    err = (got.double() - expect).abs().amax(dim=1) / scale
+    assert bool(torch.isfinite(err).all()), f"{what}: not finite"
+    bad = torch.nonzero(err > tol)
+    assert bad.numel() == 0, f"{what}: first wrong row {int(bad[0])}: {float(err[int(bad[0])]):.3e} of the logit scale (tolerance {tol:.0e})"
+    return float(err.max())
+
+
+def prompt_tokens(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, CFG["vocab_size"], (n,), generator=g).tolist()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_prompt_then_tail_through_the_captured_graph(model, dtype):
+    from mini_inference_engine_amd.engine.batch import StepRow
+    tol = F32_TOL if dtype == "float32" else BF16_TOL
+    toks = prompt_tokens(PROMPT, 31)
+    expect = plain_logits(model, dtype, toks)
+    runner = make_runner(model, dtype, pages=2 * (PROMPT // 16 + 2) + 1, max_rows=4)
+
+    rc = runner.cache.open("whole")
+    assert runner.cache.reserve(rc, 0, PROMPT)
+    got = runner.forward_step([StepRow(rc, toks, 0, list(range(PROMPT)))])
+    w = worst_error(got, expect, tol, f"{dtype}: whole prompt")
+    runner.cache.close(rc)
+
+    runner.capture_decode_graphs((1,))
+    rc = runner.cache.open("tail")
+    head = PROMPT - TAIL
+    assert runner.cache.reserve(rc, 0, head)
+    got = runner.forward_step([StepRow(rc, toks[:head], 0, [head - 1])])
+    assert not runner.last_step_captured
+    rows = [got[0].clone()]
+    for p in range(head, PROMPT):
+        assert runner.cache.reserve(rc, p, 1)
+        out = runner.forward_step([StepRow(rc, toks[p:p + 1], p, [0])])
+        assert runner.last_step_captured, "a single-token step did not go through the captured graph"
+        rows.append(out[0].clone())
+    w2 = worst_error(torch.stack(rows), expect[head - 1:], tol, f"{dtype}: tail through the graph")
+    runner.cache.close(rc)
+    runner.cache.check()
+    print(f"{dtype}: whole {w:.2e}, tail through the graph {w2:.2e} of the logit scale")
+
+
+@pytest.mark.parametrize("captured", [False, True], ids=["eager", "graphs"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_of_40_and_64_rows(model, dtype, captured):
+    """64 requests of 8 to 71 tokens.  All but their last two tokens go in as prompts (several a step);
+    then one step of 40 single-token rows and one of 64."""
+    from mini_inference_engine_amd.engine.batch import StepRow
+    tol = F32_TOL if dtype == "float32" else BF16_TOL
+    lengths = [8 + (i * 37) % 64 for i in range(64)]
+    requests = [prompt_tokens(n, 100 + i) for i, n in enumerate(lengths)]
+    runner = make_runner(model, dtype, pages=sum(-(-n // 16) for n in lengths) + 1)
+    if captured:
+        runner.capture_decode_graphs((48, 64))
+    caches = [runner.cache.open(i) for i in range(64)]
+    fed = [0] * 64
+
+    def feed(which, counts, want_last):
+        rows = []
+        for i, n in zip(which, counts):
+            assert runner.cache.reserve(caches[i], fed[i], n)
+            rows.append(StepRow(caches[i], requests[i][fed[i]:fed[i] + n], fed[i], [n - 1] if want_last else []))
+        out = runner.forward_step(rows)
+        for i, n in zip(which, counts):
+            fed[i] += n
+        return out
+
+    batch, room = [], 512
+    for i, n in enumerate(lengths):                      # prompts, as many a step as fit 512 tokens
+        if n - 2 > room:
+            feed(batch, [lengths[j] - 2 for j in batch], False)
+            batch, room = [], 512
+        batch.append(i)
+        room -= n - 2
+    feed(batch, [lengths[j] - 2 for j in batch], False)
+    assert not runner.last_step_captured
+
+    got = {}
+    out = feed(range(40), [1] * 40, True)
+    assert runner.last_step_captured == captured
+    for k, i in enumerate(range(40)):
+        got[(i, fed[i] - 1)] = out[k].clone()
+    out = feed(range(64), [1] * 64, True)
+    assert runner.last_step_captured == captured
+    for k, i in enumerate(range(64)):
+        got[(i, fed[i] - 1)] = out[k].clone()
+
+    worst = 0.0
+    for i in range(64):
+        expect = plain_logits(model, dtype, requests[i])
+        for (j, p), row in got.items():
+            if j == i:
+                worst = max(worst, worst_error(row[None], expect[p:p + 1], tol,
+                                               f"{dtype}/{'graphs' if captured else 'eager'}: request {i} position {p}",
+                                               scale=float(expect.abs().max())))
+    for rc in caches:
+        runner.cache.close(rc)
+    runner.cache.check()
+    print(f"{dtype}/{'graphs' if captured else 'eager'}: 40- and 64-row steps, worst {worst:.2e} of the logit scale")

@@ -103,6 +103,32 @@ def test_replay_gpu(tiny_models, tmp_path, name, dtype, family):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("family", ["decode_tail", "mixed"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_replay_through_captured_graphs(tiny_models, tmp_path, name, dtype, family):
+    """The same traces with every step of single-token entries replayed from a captured graph, as generation
+    runs them: static bound on the context, rows padded to the captured batch size with scratch rows."""
+    m = tiny_models[name]
+    prompts = trace_util.random_prompts(m["cfg"]["vocab_size"], LENGTHS[name], seed=11)
+    steps = make_steps(family, prompts)
+    peak = trace_util.live_token_peak(steps)
+    folder = m["folder_f32"] if dtype == "float32" else m["folder_bf16"]
+    runner = ModelRunner(folder, dtype=dtype, device="cuda", num_pages=peak // 16 + 1, max_rows=8,
+                         max_step_tokens=max(64, peak))
+    runner.capture_decode_graphs((1, 2, 4))
+    replays = []
+    run = runner.graphs.run
+    runner.graphs.run = lambda rows: (replays.append(len(rows)), run(rows))[1]
+    run_replay(runner, steps, str(tmp_path))
+    single = [len(s["entries"]) for s in steps if all(len(e["tokens"]) == 1 for e in s["entries"])]
+    assert replays == single and len(single) >= 12, "steps of single tokens must all have been replayed from graphs"
+    got = trace_util.read_outputs(str(tmp_path), steps, m["cfg"]["vocab_size"])
+    exp = expected_logits(m, prompts, bf16_weights=dtype == "bfloat16")
+    trace_util.compare(got, exp, F32_TOL if dtype == "float32" else BF16_TOL, f"{name}/{family}/{dtype}/graphs")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_cuts_agree_with_each_other(tiny_models, tmp_path, dtype):
     """The same position through four different cuts: in float32 the kernels are batch
@@ -130,8 +156,9 @@ def test_cuts_agree_with_each_other(tiny_models, tmp_path, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_trace_run_program(tiny_models, tmp_path, dtype):
+def test_trace_run_program(tiny_models, tmp_path, dtype, graphs):
     """bin/trace_run as a user calls it: a subprocess, steps on stdin, 'done' lines, files."""
     m = tiny_models["A"]
     prompts = trace_util.random_prompts(256, [5, 17, 33, 40], seed=3)
@@ -140,7 +167,7 @@ def test_trace_run_program(tiny_models, tmp_path, dtype):
     folder = m["folder_f32"] if dtype == "float32" else m["folder_bf16"]
     out = str(tmp_path / "out")
     proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-                           "--out", out, "--max-tokens", str(peak)],
+                           "--out", out, "--max-tokens", str(peak)] + (["--hip-graphs"] if graphs else []),
                           input="\n".join(trace_util.to_lines(steps)) + "\n", capture_output=True, text=True,
                           timeout=600)
     assert proc.returncode == 0, proc.stderr[-2000:]
