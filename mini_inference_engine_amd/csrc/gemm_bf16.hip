@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(WAVES * 64)
 skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict__ W, long ldw, void* __restrict__ outv,
                    long ldo, int M, int N, int K, int up_offset, RopeArgs rope, NormArgs nf) {
   // k-steps per group of loads (two groups are in flight per wave)
-  constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
+  constexpr int U = MT == 1 ? 4 : 2;
   constexpr int SG_WAVES = WAVES;
   constexpr int SG_THREADS = WAVES * 64;
   constexpr int PER = (MT * 256 + SG_THREADS - 1) / SG_THREADS;   // results (m, n) a thread owns after the reduction

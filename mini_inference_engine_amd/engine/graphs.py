@@ -10,6 +10,7 @@ upload.  No memset node is recorded: buffers are cleared by kernels.
 """
 from __future__ import annotations
 
+import gc
 import time
 
 import torch
@@ -17,7 +18,9 @@ import torch
 
 class DecodeGraphs:
     def __init__(self, runner, batch_sizes, verbose: bool = True):
-        self.runner = runner
+        # The runner owns this object, so it is not kept here: a reference back would make a cycle, and the
+        # graphs with all they hold would then be freed whenever the collector runs, possibly in the middle
+        # of a later capture, which the runtime does not survive.  ``run`` takes the runner instead.
         arena = runner.arena
         self.sizes = sorted(b for b in set(batch_sizes) if 0 < b <= arena.max_rows and b <= arena.max_tokens)
         self.graphs = {}
@@ -31,8 +34,16 @@ class DecodeGraphs:
             runner.model.forward(step)                  # loads libraries, warms the allocator
             torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, pool=pool):
-                logits = runner.model.forward(step)
+            # no garbage collection while the stream records: a collected object that owns device memory
+            # or another graph would free it in the middle of the capture
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(g, pool=pool):
+                    logits = runner.model.forward(step)
+            finally:
+                if collecting:
+                    gc.enable()
             pool = g.pool()
             self.graphs[bs] = (g, logits)
         torch.cuda.synchronize()
@@ -43,11 +54,11 @@ class DecodeGraphs:
     def fits(self, rows: int) -> bool:
         return bool(self.sizes) and rows <= self.sizes[-1]
 
-    def run(self, rows) -> torch.Tensor | None:
+    def run(self, runner, rows) -> torch.Tensor | None:
         """``rows``: single-token StepRows.  Logits of the rows that want them, in order."""
         bs = next(s for s in self.sizes if s >= len(rows))
         picked = [i for i, r in enumerate(rows) if len(r.want)]
-        self.runner.build(rows, pad_rows_to=bs, static_context=self.static_context, want_all=True)
+        runner.build(rows, pad_rows_to=bs, static_context=self.static_context, want_all=True)
         g, logits = self.graphs[bs]
         g.replay()
         if not picked:

@@ -111,7 +111,7 @@ class ModelRunner:
         self.last_step_captured = False
         if self.graphs is not None and self.graphs.fits(len(rows)) and all(len(r.tokens) == 1 for r in rows):
             self.last_step_captured = True
-            return self.graphs.run(rows)
+            return self.graphs.run(self, rows)
         step = self.build(rows)
         return self.model.forward(step)
 

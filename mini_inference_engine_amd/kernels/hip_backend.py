@@ -50,69 +50,18 @@ class HipBackend(KernelBackend):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU visible to torch: the engine needs an MI355X (gfx950)")
         self._libs = {}
+        self._zeros = None          # 256 zero bytes on the device, what masked loads of the mid-row product read
         self.true_fp32 = act_dtype == torch.float32
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
 
     # ------------------------------------------------------------ plumbing
     def lib(self, module: str, defines: tuple = ()):
+        """The loaded library of a registered kernel module (library.register_kernel_module), entry points
+        declared with the argument types it was registered with."""
         key = (module, defines)
         if key not in self._libs:
-            lib = library.load(module, defines)
-            self._declare(module, lib)
-            self._libs[key] = lib
+            self._libs[key] = library.load(module, defines)
         return self._libs[key]
-
-    @staticmethod
-    def _declare(module: str, lib) -> None:
-        sig = {
-            "embed_norm": {
-                "mie_embedding": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
-                "mie_add_rmsnorm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
-                                    c_int, c_float, c_void_p],
-            },
-            "rope_kv": {
-                "mie_rotary_kv_store": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                        c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
-            },
-            "gemm": {
-                "mie_gemm_nt": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_void_p,
-                                c_int, c_int, c_int, c_void_p],
-                "mie_silu_mul": [c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
-            },
-            "attention": {
-                "mie_paged_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
-                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                        c_void_p],
-            },
-            "sampling": {
-                "mie_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
-            },
-            "gemm_bf16": {
-                "mie_skinny_gemm": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_int,
-                                    c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p,
-                                    c_void_p],
-                "mie_skinny_qkv_rope": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p,
-                                        c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                        c_void_p, c_int, c_float, c_void_p],
-                "mie_skinny_max_rows": [],
-            },
-            "attention_bf16": {
-                "mie_decode_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                         c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                                         c_int, c_void_p],
-                "mie_decode_block_keys": [],
-                "mie_attention_bf16_head_dim": [],
-            },
-            "prefill_attention_bf16": {
-                "mie_prefill_attention": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                          c_void_p],
-            },
-        }.get(module, {})
-        for name, argtypes in sig.items():
-            fn = getattr(lib, name)
-            fn.argtypes = argtypes
-            fn.restype = c_int
 
     def _stream(self) -> c_void_p:
         # the handle alone: building torch's Stream object costs several microseconds a launch
@@ -214,6 +163,52 @@ class HipBackend(KernelBackend):
                                                M, n_out, w.shape[1], *norm_args, self._stream()))
         return made
 
+    # ---- products of 33 to 128 rows on a narrow weight: split over K, partial results, one kernel that adds
+    # them up and does what follows the product
+    MID_MAX_ROWS = 128
+    MID_MAX_COLS = 4096        # wider weights have tiles enough for the library product without a split of K
+    RED_BF16, RED_F32, RED_ADD, RED_ADD_NORM = 0, 1, 2, 3
+
+    def _mid_ok(self, x, w, bias) -> bool:
+        """Whether the split product takes x w^T: 33 to 64 rows, or up to 128 where K is long (measured at the
+        benchmark's shapes: beyond 64 rows the library product with its separate epilogue kernel is as fast
+        unless K >= 4096)."""
+        M = x.shape[0]
+        most = self.MID_MAX_ROWS if w.shape[1] >= 4096 else min(64, self.MID_MAX_ROWS)
+        return (not self.true_fp32 and bias is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+                and self.SKINNY_MAX_ROWS < M <= most and w.shape[0] <= self.MID_MAX_COLS
+                and w.shape[0] % 4 == 0 and w.shape[1] % 8 == 0 and w.stride(0) % 8 == 0 and x.stride(0) % 8 == 0
+                and w.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0)
+
+    @staticmethod
+    def mid_splits(N: int, K: int) -> int:
+        """Splits of K wanted for a weight [N, K]: enough for 256 workgroups of 64 weight rows, each split
+        at least 256 wide.  A function of the weight's shape alone: a row's sums do not depend on its batch."""
+        tiles = -(-N // 64)
+        return max(1, min(8, 256 // tiles, K // 256))
+
+    def _mid_partials(self, x, w):
+        """part [splits, M, N] float32 of x w^T."""
+        lib = self.lib("gemm_mid_bf16")
+        M, K = x.shape
+        N = w.shape[0]
+        wanted = self.mid_splits(N, K)
+        splits = lib.mie_mid_splits(K, wanted)
+        part = torch.empty((splits, M, N), dtype=torch.float32, device=w.device)
+        if self._zeros is None:
+            self._zeros = torch.zeros(64, dtype=torch.int32, device=w.device)
+        library.check(lib, lib.mie_mid_gemm(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(part), M, N, K, wanted,
+                                            _ptr(self._zeros), self._stream()))
+        return part
+
+    def _mid_reduce(self, part, mode, out=None, stream=None, g=None, x_next=None, eps=0.0):
+        lib = self.lib("gemm_mid_bf16")
+        splits, M, N = part.shape
+        library.check(lib, lib.mie_mid_reduce(
+            _ptr(part), splits, M, N, mode, _ptr(out), out.stride(0) if out is not None else 0, _ptr(stream), _ptr(g),
+            int(g is not None and g.dtype == torch.float32), _ptr(x_next), x_next.stride(0) if x_next is not None else 0,
+            float(eps), self._stream()))
+
     def linear(self, x, w, bias=None, out_dtype=None, add_to=None):
         self._on_device(w, bias)
         _rows_ok(w, "linear: w")
@@ -247,6 +242,21 @@ class HipBackend(KernelBackend):
             out = torch.empty((M, N), dtype=out_dtype, device=w.device)
             self._skinny(x, w, self.EPI_BF16 if out_dtype == torch.bfloat16 else self.EPI_F32, out, N)
             return out
+        if self._mid_ok(x, w, bias) and out_dtype in (torch.bfloat16, torch.float32):
+            part = self._mid_partials(x, w)
+            if sink is None:
+                out = torch.empty((M, N), dtype=out_dtype, device=w.device)
+                self._mid_reduce(part, self.RED_BF16 if out_dtype == torch.bfloat16 else self.RED_F32, out=out)
+                return out
+            g = sink.norm_weight
+            if g is None or g.dtype not in (torch.bfloat16, torch.float32) or tuple(g.shape) != (N,) or not g.is_contiguous():
+                self._mid_reduce(part, self.RED_ADD, stream=sink.stream)
+                return None
+            normed = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+            self._mid_reduce(part, self.RED_ADD_NORM, stream=sink.stream, g=g, x_next=normed, eps=sink.norm_eps)
+            done = Normed(self, None, sink.stream, g, sink.norm_eps)
+            done._value = normed            # the norm is computed: materialize() hands this out
+            return done
         if not self.true_fp32 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
             # library matrix product, 32-bit accumulation, as the reference's F.linear.  What goes into the
             # float32 stream or out as logits leaves the product in float32: the sums are not rounded to
@@ -298,24 +308,15 @@ class HipBackend(KernelBackend):
         elif isinstance(x, Normed):
             x = x.materialize()
         fused = can_rope and self._skinny_ok(x, w_qkv, None)
+        if not fused and can_rope and self._mid_ok(x, w_qkv, None) and self.act_dtype == torch.bfloat16:
+            return self._mid_rotary_kv_store(x, w_qkv, positions, cos, sin, Hq, Hkv, D, k_cache, v_cache, slot_mapping)
         if not fused:
             return super().linear_rotary_kv_store(x, w_qkv, positions, cos, sin, rotary_dim, Hq, Hkv, D, k_cache,
                                                   v_cache, slot_mapping)
         self._on_device(x, w_qkv, positions, cos, sin, k_cache, v_cache, slot_mapping)
         M, K = x.shape
-        if tuple(w_qkv.shape) != ((Hq + 2 * Hkv) * D, K):
-            raise ValueError(f"linear_rotary_kv_store: w {tuple(w_qkv.shape)} for {Hq}+2x{Hkv} heads of {D}, K {K}")
-        page = k_cache.shape[2]
-        for name, t, want in (("k_cache", k_cache, (k_cache.shape[0], Hkv, page, D)),
-                              ("v_cache", v_cache, (k_cache.shape[0], Hkv, D, page))):
-            if tuple(t.shape) != want or t.dtype != torch.bfloat16 or not t.is_contiguous():
-                raise ValueError(f"linear_rotary_kv_store: {name} {tuple(t.shape)} {t.dtype}, expected {want}")
-        for name, t in (("cos", cos), ("sin", sin)):
-            if t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != D // 2 or not t.is_contiguous():
-                raise ValueError(f"linear_rotary_kv_store: {name} must be contiguous float32 [positions, {D // 2}]")
-        for name, t in (("positions", positions), ("slot_mapping", slot_mapping)):
-            if t.dtype != torch.int32 or t.shape[0] != M or not t.is_contiguous():
-                raise ValueError(f"linear_rotary_kv_store: {name} must be contiguous int32 [{M}]")
+        page = self._check_rope_operands("linear_rotary_kv_store", M, K, w_qkv, positions, cos, sin, Hq, Hkv, D,
+                                         k_cache, v_cache, slot_mapping)
         q = torch.empty((M, Hq * D), dtype=torch.bfloat16, device=x.device)
         lib = self.lib("gemm_bf16")
         library.check(lib, lib.mie_skinny_qkv_rope(
@@ -323,6 +324,37 @@ class HipBackend(KernelBackend):
             _ptr(sin), _ptr(slot_mapping), _ptr(k_cache), _ptr(v_cache), M, Hq, Hkv, D, page, K,
             _ptr(prepared["ss"]) if prepared else None, prepared["tiles"] if prepared else 0, float(eps),
             self._stream()))
+        return q
+
+    def _check_rope_operands(self, what, M, K, w_qkv, positions, cos, sin, Hq, Hkv, D, k_cache, v_cache, slot_mapping):
+        if tuple(w_qkv.shape) != ((Hq + 2 * Hkv) * D, K):
+            raise ValueError(f"{what}: w {tuple(w_qkv.shape)} for {Hq}+2x{Hkv} heads of {D}, K {K}")
+        page = k_cache.shape[2]
+        for name, t, want in (("k_cache", k_cache, (k_cache.shape[0], Hkv, page, D)),
+                              ("v_cache", v_cache, (k_cache.shape[0], Hkv, D, page))):
+            if tuple(t.shape) != want or t.dtype != torch.bfloat16 or not t.is_contiguous():
+                raise ValueError(f"{what}: {name} {tuple(t.shape)} {t.dtype}, expected {want}")
+        for name, t in (("cos", cos), ("sin", sin)):
+            if t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != D // 2 or not t.is_contiguous():
+                raise ValueError(f"{what}: {name} must be contiguous float32 [positions, {D // 2}]")
+        for name, t in (("positions", positions), ("slot_mapping", slot_mapping)):
+            if t.dtype != torch.int32 or t.shape[0] != M or not t.is_contiguous():
+                raise ValueError(f"{what}: {name} must be contiguous int32 [{M}]")
+        return page
+
+    def _mid_rotary_kv_store(self, x, w_qkv, positions, cos, sin, Hq, Hkv, D, k_cache, v_cache, slot_mapping):
+        """The q/k/v projection of 33 to 128 rows: split product, then one kernel that adds the partial
+        results, rotates q and k and writes k and v to the cache.  Returns q [M, Hq * D]."""
+        self._on_device(x, w_qkv, positions, cos, sin, k_cache, v_cache, slot_mapping)
+        M, K = x.shape
+        page = self._check_rope_operands("linear_rotary_kv_store", M, K, w_qkv, positions, cos, sin, Hq, Hkv, D,
+                                         k_cache, v_cache, slot_mapping)
+        part = self._mid_partials(x, w_qkv)
+        q = torch.empty((M, Hq * D), dtype=torch.bfloat16, device=x.device)
+        lib = self.lib("gemm_mid_bf16")
+        library.check(lib, lib.mie_mid_reduce_rope_kv(
+            _ptr(part), part.shape[0], M, _ptr(q), q.stride(0), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
+            _ptr(k_cache), _ptr(v_cache), Hq, Hkv, D, page, self._stream()))
         return q
 
     def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,

@@ -24,14 +24,41 @@ import time
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 ARCH = "gfx950"
-MODULES = ("embed_norm", "rope_kv", "gemm", "attention", "sampling", "gemm_bf16", "attention_bf16",
-           "prefill_attention_bf16")
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-fno-gpu-sanitize",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-# Per module, beside FLAGS.  prefill_attention_bf16: matrix instructions keep their accumulators in
-# ordinary vector registers; otherwise the compiler parks the outputs in accumulation registers and copies
-# all of them back and forth around every key block for the sake of the (rare) rescaling.
-MODULE_FLAGS = {"prefill_attention_bf16": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
+class KernelModule:
+    """One HIP source that becomes one shared library (per variant).  ``signatures``: entry point ->
+    ctypes argument types (every entry point returns int: 0, or a negative code with a message readable
+    through <name>_last_error()).  ``variants``: lists of -D defines built ahead of time; others compile at
+    first use.  ``flags``: compiler flags beside FLAGS.  ``source``: the .hip file (by default csrc/<name>.hip);
+    a module outside the package hashes its own file and this package's headers."""
+
+    def __init__(self, name, signatures=None, variants=None, flags=None, source=None):
+        self.name = name
+        self.signatures = dict(signatures or {})
+        self.variants = [tuple(v) for v in (variants or [()])]
+        self.flags = list(flags or [])
+        self.source = source or os.path.join(CSRC, name + ".hip")
+
+
+MODULES: dict[str, KernelModule] = {}
+
+
+def register_kernel_module(name: str, signatures=None, variants=None, flags=None, source=None) -> KernelModule:
+    """Make a kernel source known to the loader, the build-everything step and the backend's
+    declaration of argument types.  A part that brings a kernel of its own calls this (from outside the
+    package too) and then reaches its entry points through ``HipBackend.lib(name)``."""
+    MODULES[name] = KernelModule(name, signatures, variants, flags, source)
+    return MODULES[name]
+
+
+def kernel_module(name: str) -> KernelModule:
+    if name not in MODULES:
+        raise KernelLibraryError(f"kernel module {name!r} is not registered (known: {sorted(MODULES)})")
+    return MODULES[name]
+
 
 _loaded: dict = {}
 _lock = threading.Lock()
@@ -42,15 +69,16 @@ class KernelLibraryError(RuntimeError):
 
 
 def available_modules() -> list[str]:
-    return [m for m in MODULES if os.path.isfile(os.path.join(CSRC, m + ".hip"))]
+    return [name for name, m in MODULES.items() if os.path.isfile(m.source)]
 
 
-def _digest(module: str, defines: tuple) -> str:
+def _digest(name: str, defines: tuple) -> str:
+    mod = kernel_module(name)
     h = hashlib.sha256()
-    for fn in [module + ".hip"] + sorted(f for f in os.listdir(CSRC) if f.endswith(".hpp")):
-        with open(os.path.join(CSRC, fn), "rb") as f:
+    for path in [mod.source] + sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")):
+        with open(path, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS + MODULE_FLAGS.get(module, []) + [ARCH] + list(defines)).encode())
+    h.update(" ".join(FLAGS + mod.flags + [ARCH] + list(defines)).encode())
     return h.hexdigest()[:16]
 
 
@@ -87,7 +115,8 @@ def _hipcc() -> str:
 
 def build(module: str, defines: tuple = (), verbose: bool = True) -> str:
     """Compile one module now (also when a built file is already there)."""
-    src = os.path.join(CSRC, module + ".hip")
+    mod = kernel_module(module)
+    src = mod.source
     if not os.path.isfile(src):
         raise KernelLibraryError(f"no kernel source {src}")
     name = library_file(module, defines)
@@ -106,7 +135,7 @@ def build(module: str, defines: tuple = (), verbose: bool = True) -> str:
         raise KernelLibraryError(f"no writable folder to build kernels in (tried {_build_dirs()})")
     out = os.path.join(out_dir, name)
     tmp = os.path.join(out_dir, f".{name}.{os.getpid()}.{threading.get_ident()}.tmp")
-    cmd = [_hipcc(), f"--offload-arch={ARCH}", *FLAGS, *MODULE_FLAGS.get(module, []), *defines, "-I", CSRC, src, "-o", tmp]
+    cmd = [_hipcc(), f"--offload-arch={ARCH}", *FLAGS, *mod.flags, *defines, "-I", CSRC, src, "-o", tmp]
     env = dict(os.environ)
     env.setdefault("HOME", out_dir)        # hipcc's helpers want some HOME; an empty one is fine
     t0 = time.time()
@@ -164,6 +193,10 @@ def load(module: str, defines: tuple = ()) -> ctypes.CDLL:
         err.restype = ctypes.c_char_p
         lib._mie_error = err
         lib._mie_path = path
+        for entry, argtypes in kernel_module(module).signatures.items():
+            fn = getattr(lib, entry)
+            fn.argtypes = list(argtypes)
+            fn.restype = ctypes.c_int
         _loaded[key] = lib
         return lib
 
@@ -179,15 +212,14 @@ def build_all(verbose: bool = True, jobs: int = 4) -> list[str]:
         return list(ex.map(lambda w: build(w[0], w[1], verbose), work))
 
 
-def variants_of(module: str) -> list[tuple]:
-    """Compile-time variants of a module; plain modules have one (no defines)."""
-    try:
-        from . import variants
-        return variants.VARIANTS.get(module, [()])
-    except ImportError:
-        return [()]
+def variants_of(name: str) -> list[tuple]:
+    """Compile-time variants of a module built ahead of time; plain modules have one (no defines)."""
+    return list(kernel_module(name).variants)
 
 
 def check(lib, code: int) -> None:
     if code != 0:
         raise RuntimeError(lib._mie_error().decode(errors="replace"))
+
+
+from . import modules as _builtin_modules  # noqa: E402,F401  (registers the package's own kernel modules)

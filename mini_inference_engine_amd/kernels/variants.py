@@ -6,8 +6,3 @@ up to 256) gets its variant compiled at first use.
 """
 
 HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
-
-VARIANTS = {
-    "attention_bf16": [(f"-DHEAD_DIM={d}",) for d in HEAD_DIMS],
-    "prefill_attention_bf16": [(f"-DHEAD_DIM={d}",) for d in HEAD_DIMS],
-}

@@ -172,6 +172,99 @@ def test_skinny_linear(ops, shape):
     torch.testing.assert_close(stream, expect, atol=2e-3, rtol=2e-3)
 
 
+# --------------------------------------------------- products of 33 to 128 rows (bfloat16), split over K
+@pytest.fixture(scope="module")
+def engine_ops():
+    """The backend with the engine's own thresholds between its three product paths."""
+    from mini_inference_engine_amd.kernels.hip_backend import HipBackend
+    return HipBackend(torch.bfloat16, DEV)
+
+
+MID_SHAPES = [(33, 2048, 2048), (64, 2048, 2560), (128, 5632, 2048), (50, 2008, 1000), (37, 256, 64), (100, 4104, 4096),
+              (65, 4096, 4), (40, 4096, 2048), (48, 8, 4)]
+
+
+@pytest.mark.parametrize("shape", MID_SHAPES)
+def test_mid_linear(engine_ops, shape):
+    M, K, N = shape
+    o = engine_ops
+    torch.manual_seed(M * 5 + N)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    assert o._mid_ok(x, w, None) and not o._skinny_ok(x, w, None), "this shape must take the split product"
+    exact = x.double() @ w.double().T
+    y32 = o.linear(x, w, out_dtype=torch.float32)
+    torch.testing.assert_close(y32.double(), exact, atol=1e-4, rtol=1e-4)        # float32 sums of exact products
+    y = o.linear(x, w)
+    assert y.dtype == torch.bfloat16
+    torch.testing.assert_close(y.float(), exact.float(), atol=2e-2, rtol=1e-2)
+    # a row's result does not depend on the rows beside it, nor on the number of row tiles
+    for a, b in ((0, 33), (M - 33, M), (0, min(M, 64))):
+        assert torch.equal(o.linear(x[a:b].contiguous(), w, out_dtype=torch.float32), y32[a:b])
+    most = 128 if K >= 4096 else 64
+    big = torch.cat([x, x[:most - M]]) if M < most else x
+    assert torch.equal(o.linear(big, w, out_dtype=torch.float32)[:M], y32)
+    # residual add
+    stream = torch.randn(M, N, device=DEV)
+    expect = stream.double() + exact
+    assert o.linear(x, w, add_to=stream) is None
+    torch.testing.assert_close(stream.double(), expect, atol=1e-4, rtol=1e-4)
+    # residual add and the norm that reads the stream next, float32 and bfloat16 norm weights
+    from mini_inference_engine_amd.kernels.api import Normed, Sink
+    for gdt in (torch.float32, torch.bfloat16):
+        stream = torch.randn(M, N, device=DEV)
+        g = (1 + 0.1 * torch.randn(N, device=DEV)).to(gdt)
+        r = stream.double() + exact
+        want = r * torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + 1e-5) * g.double()
+        out = o.linear(x, w, add_to=Sink(stream, g, 1e-5))
+        assert isinstance(out, Normed) and out.pending is None and out.weight is g
+        torch.testing.assert_close(stream.double(), r, atol=1e-4, rtol=1e-4)
+        torch.testing.assert_close(out.materialize().double(), want, atol=2e-2, rtol=1e-2)
+
+
+def test_mid_linear_refuses_what_it_cannot_run(engine_ops):
+    o = engine_ops
+    lib = o.lib("gemm_mid_bf16")
+    x = torch.zeros(200, 64, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(64, 64, device=DEV, dtype=torch.bfloat16)
+    part = torch.zeros(1, 200, 64, device=DEV)
+    z = torch.zeros(64, dtype=torch.int32, device=DEV)
+    assert lib.mie_mid_gemm(x.data_ptr(), 64, w.data_ptr(), 64, part.data_ptr(), 200, 64, 64, 1, z.data_ptr(), None) != 0
+    assert b"at most 128" in lib._mie_error()
+    assert lib.mie_mid_gemm(x.data_ptr(), 60, w.data_ptr(), 60, part.data_ptr(), 40, 64, 60, 1, z.data_ptr(), None) != 0
+    assert b"multiple of 8" in lib._mie_error()
+    assert lib.mie_mid_reduce(part.data_ptr(), 1, 40, 66, 1, part.data_ptr(), 66, None, None, 0, None, 0, 0.0, None) != 0
+    assert b"width" in lib._mie_error()
+    assert not o._mid_ok(x[:40], torch.zeros(8192, 64, device=DEV, dtype=torch.bfloat16), None), "wide weights go to the library"
+
+
+@pytest.mark.parametrize("geom", [(2, 1, 16), (3, 1, 32), (4, 2, 48), (32, 4, 64), (5, 5, 96), (8, 2, 128), (2, 1, 256)])
+@pytest.mark.parametrize("M", [40, 64])
+def test_mid_projection_rotary_store(engine_ops, geom, M):
+    """Split projection, then one kernel for sum + rotary + cache write, against the separate references."""
+    from mini_inference_engine_amd.parts.rope import rotary_tables
+    Hq, Hkv, D = geom
+    o = engine_ops
+    torch.manual_seed(D + M)
+    K, page, pages = 264, 16, 12
+    cos, sin = (t.to(DEV) for t in rotary_tables(10000.0, D, 300))
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn((Hq + 2 * Hkv) * D, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    assert o._mid_ok(x, w, None)
+    pos = torch.randint(0, 300, (M,), device=DEV, dtype=torch.int32)
+    slots = (torch.randperm((pages - 1) * page, device=DEV)[:M] + page).to(torch.int32)
+    kc, vc = make_cache(pages, Hkv, page, D, torch.bfloat16)
+    kc_ref, vc_ref = kc.float(), vc.float()
+    qkv_ref = ref.ref_linear(x, w, None, torch.float32)
+    ref.ref_rotary_kv_store(qkv_ref, pos, cos, sin, D, Hq, Hkv, D, kc_ref, vc_ref, slots)
+    out = o.linear_rotary_kv_store(x, w, pos, cos, sin, D, Hq, Hkv, D, kc, vc, slots)
+    assert tuple(out.shape) == (M, Hq * D), "q alone comes back"
+    torch.testing.assert_close(out.float(), qkv_ref[:, :Hq * D], atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(kc.float(), kc_ref, atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(vc.float(), vc_ref, atol=2e-2, rtol=1e-2)
+    assert torch.equal(kc[0].float(), kc_ref[0]) and torch.equal(vc[0].float(), vc_ref[0]), "untouched pages stay untouched"
+
+
 def test_lazy_norm_input_adds_once(ops):
     """A Normed handed to linear: what is pending is added to the stream exactly once, however often it is used."""
     o = ops[torch.bfloat16]
