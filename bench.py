@@ -1,6 +1,8 @@
-"""Decode and prefill throughput of the engine at TinyLlama-1.1B layer sizes, random weights.
+"""Decode and prefill throughput of the engine at TinyLlama-1.1B layer sizes (or, with --shape, at those of
+Llama-2-7B or Llama-3-8B), random weights.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--shape tinyllama] [--context N] [--layers L]
+    python bench.py --kernels [--shape ...] [--batch 8] [--context N]     each dominant kernel alone
 
 A step is one decode step of the engine (schedule, batch, captured forward, sampling,
 bookkeeping: LLMEngine.step, the call a user's loop makes; it starts a step and reads the tokens
@@ -8,11 +10,16 @@ of the one before, so K calls between two synchronisations are K whole steps), a
 reference's benchmarks/bench_latency.py:33-49: prefill ``batch`` equal prompts, warm up,
 time K steps between device synchronisations.  Prints one JSON line:
   value     decoded tokens a second at ``batch`` (default 8) with contexts just below ``context``
-  points    the same at batch 1 and 64; output and total tokens a second of the reference's mixed
-            end-to-end workload (256 requests at once, prompts of 128..512 and outputs of 64..512 tokens)
+  points    the same at batch 1 and 64, and at ``batch`` with contexts of 512; output and total tokens a second
+            of the reference's mixed end-to-end workload (256 requests at once, prompts of 128..512 and outputs
+            of 64..512 tokens; TinyLlama sizes only)
   prefill   one 2,048-token prompt in one step: tokens a second, and flops / time / peak
   roofline  bytes a decode step must read (weights once + live cache) / time, against HBM peak
 Peaks: MI355X HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
+With --kernels no engine runs: the kernels a decode step and a prefill spend their time in are launched
+alone (captured in a graph, over rotating weight buffers so that nothing stays cached), and one JSON line
+lists for each its time, the bytes or flops it has to move or do and that over time over the peak
+(the reference's benchmarks/bench_kernels.py:1-79 does the same for its kernels, in GB/s).
 The engine runs on one GPU; for --gpus > 1 one line says so and the exit code is 2.
 """
 from __future__ import annotations
@@ -33,13 +40,23 @@ FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 REFERENCE_B8_TOKENS_PER_S = 8 / 10.02e-3
 
 
+SHAPE_NAMES = {"tinyllama": "TinyLlama-1.1B", "llama2-7b": "Llama-2-7B", "llama3-8b": "Llama-3-8B"}
+
+
+def shape_config(shape: str = "tinyllama", layers: int | None = None):
+    """Layer sizes by name (the command line's table); ``layers``: fewer layers than the model has."""
+    from mini_inference_engine_amd.__main__ import SHAPES
+    from mini_inference_engine_amd.config import LlamaConfig
+    d = dict(SHAPES[shape], architectures=["LlamaForCausalLM"], eos_token_id=2)
+    full = d["num_hidden_layers"]
+    if layers:
+        d["num_hidden_layers"] = layers
+    return LlamaConfig.from_dict(d), full
+
+
 def tinyllama_config(layers: int | None = None):
     """TinyLlama-1.1B layer sizes, the configuration the benchmark is quoted on."""
-    from mini_inference_engine_amd.config import LlamaConfig
-    return LlamaConfig(vocab_size=32000, hidden_size=2048, intermediate_size=5632,
-                       num_hidden_layers=layers or 22, num_attention_heads=32, num_key_value_heads=4, head_dim=64,
-                       rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=2048,
-                       tie_word_embeddings=False, eos_token_id=2)
+    return shape_config("tinyllama", layers)[0]
 
 
 def linear_params(cfg) -> int:
@@ -153,14 +170,121 @@ def measure_mixed(cfg, weights, dtype, requests: int, seed: int, use_graphs: boo
             "seconds": round(best[0], 3), "steps": best[1], "preemptions": eng.scheduler.num_preemptions}
 
 
+def measure_kernels(cfg, args) -> int:
+    """Each dominant kernel alone: captured in a graph over rotating weight buffers (nothing stays cached
+    from one launch to the next), timed with events around several replays."""
+    import torch
+    from mini_inference_engine_amd.kernels.api import Sink
+    from mini_inference_engine_amd.kernels.hip_backend import HipBackend
+    from mini_inference_engine_amd.parts.rope import rotary_tables
+    from types import SimpleNamespace
+    dev = "cuda"
+    ops = HipBackend(torch.bfloat16, dev)
+    h, inter, D = cfg.hidden_size, cfg.intermediate_size, cfg.head_dim
+    Hq, Hkv, V = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.vocab_size
+    M, ctx, page = args.batch, args.context, args.block_size
+    T = min(2048, ctx)
+    copies = max(2, min(12, int(3e8 // (2 * inter * h * 2)) + 1))     # enough weight sets to exceed every cache
+
+    def timed(run, n):
+        run(0)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(n):
+                run(i)
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / (5 * n)
+
+    def weights(n_out, k):
+        return [(torch.randn(n_out, k, device=dev) * 0.02).to(torch.bfloat16) for _ in range(copies)]
+
+    out = []
+
+    def report(name, seconds, nbytes=None, flops=None):
+        r = {"kernel": name, "us": round(seconds * 1e6, 2)}
+        if nbytes is not None:
+            r.update(bytes=int(nbytes), GB_s=round(nbytes / seconds / 1e9, 1), frac_hbm=round(nbytes / seconds / HBM_PEAK, 3))
+        if flops is not None:
+            r.update(flops=int(flops), PFLOP_s=round(flops / seconds / 1e15, 3),
+                     frac_mfma=round(flops / seconds / FLOP_PEAK["bfloat16"], 3))
+        out.append(r)
+
+    # ---- the decode step's products at M rows (weights once + x + y)
+    cos, sin = (t.to(dev) for t in rotary_tables(cfg.rope_theta, D, ctx + 1))
+    pages = M * (-(-ctx // page)) + 2
+    kc = torch.randn(pages, Hkv, page, D, device=dev).to(torch.bfloat16)
+    vc = torch.randn(pages, Hkv, D, page, device=dev).to(torch.bfloat16)
+    g_norm = torch.ones(h, device=dev, dtype=torch.bfloat16)
+    x = torch.randn(M, h, device=dev).to(torch.bfloat16)
+    act = torch.randn(M, inter, device=dev).to(torch.bfloat16)
+    att = torch.randn(M, Hq * D, device=dev).to(torch.bfloat16)
+    stream = torch.randn(M, h, device=dev)
+    pos = torch.full((M,), ctx - 1, device=dev, dtype=torch.int32)
+    slots = (torch.arange(M, device=dev, dtype=torch.int32) * (-(-ctx // page)) + 1) * page + (ctx - 1) % page
+    n_qkv = (Hq + 2 * Hkv) * D
+    w = weights(n_qkv, h)
+    t = timed(lambda i: ops.linear_rotary_kv_store(x, w[i % copies], pos, cos, sin, D, Hq, Hkv, D, kc, vc, slots), copies)
+    report(f"qkv product + rotary + cache write, {M} rows", t, 2 * n_qkv * h + 2 * M * (h + n_qkv))
+    w = weights(h, Hq * D)
+    t = timed(lambda i: ops.linear(att, w[i % copies], add_to=Sink(stream, g_norm, cfg.rms_norm_eps)), copies)
+    report(f"o product + add + next norm, {M} rows", t, 2 * h * Hq * D + M * (2 * Hq * D + 8 * h + 2 * h))
+    w = weights(2 * inter, h)
+    t = timed(lambda i: ops.linear_silu_mul(x, w[i % copies], inter), copies)
+    report(f"gate/up product + SwiGLU, {M} rows", t, 2 * 2 * inter * h + 2 * M * (h + inter))
+    w = weights(h, inter)
+    t = timed(lambda i: ops.linear(act, w[i % copies], add_to=Sink(stream, g_norm, cfg.rms_norm_eps)), copies)
+    report(f"down product + add + next norm, {M} rows", t, 2 * h * inter + M * (2 * inter + 8 * h + 2 * h))
+    w = weights(V, h)[:max(2, copies // 4)]
+    t = timed(lambda i: ops.linear(x, w[i % len(w)], out_dtype=torch.float32), len(w))
+    report(f"head product, float32 logits, {M} rows", t, 2 * V * h + M * (2 * h + 4 * V))
+    del w
+    # ---- decode attention over the cache (keys and values of every row once)
+    bt = (torch.arange(M * (-(-ctx // page)), device=dev, dtype=torch.int32) + 1).view(M, -1).contiguous()
+    qkv = torch.randn(M, n_qkv, device=dev).to(torch.bfloat16)
+    step = SimpleNamespace(token_row=torch.arange(M, device=dev, dtype=torch.int32), positions=pos, num_rows=M,
+                           max_context=ctx, num_tokens=M, num_decode_rows=M, max_row_tokens=1, row_start=None,
+                           row_position=None)
+    group = SimpleNamespace(block_tables=bt, max_blocks=bt.shape[1])
+    t = timed(lambda i: ops.paged_attention(qkv, Hq, Hkv, D, kc, vc, group, step, D ** -0.5, None), 8)
+    report(f"decode attention + merge, {M} rows of {ctx} keys", t, 2 * 2 * M * ctx * Hkv * D)
+    # ---- prefill: attention over a T-token prompt, and the library product it sits between
+    qkv = torch.randn(T, n_qkv, device=dev).to(torch.bfloat16)
+    pstep = SimpleNamespace(token_row=torch.zeros(T, device=dev, dtype=torch.int32),
+                            positions=torch.arange(T, device=dev, dtype=torch.int32), num_rows=1, max_context=T,
+                            num_tokens=T, num_decode_rows=0, max_row_tokens=T,
+                            row_start=torch.tensor([0, T], device=dev, dtype=torch.int32),
+                            row_position=torch.zeros(1, device=dev, dtype=torch.int32))
+    pgroup = SimpleNamespace(block_tables=bt[:1].contiguous(), max_blocks=bt.shape[1])
+    t = timed(lambda i: ops.paged_attention(qkv, Hq, Hkv, D, kc, vc, pgroup, pstep, D ** -0.5, None), 8)
+    report(f"prefill attention, {T} tokens", t, flops=2.0 * Hq * D * T * (T + 1))
+    xt = torch.randn(T, h, device=dev).to(torch.bfloat16)
+    w = weights(2 * inter, h)
+    t = timed(lambda i: ops.linear(xt, w[i % copies]), copies)
+    report(f"gate/up product (library), {T} rows", t, flops=2.0 * T * 2 * inter * h)
+    print(json.dumps({"metric": "kernel_times", "shape": SHAPE_NAMES[args.shape], "rows": M, "context": ctx,
+                      "peaks": {"hbm_GB_s": HBM_PEAK / 1e9, "bf16_PFLOP_s": FLOP_PEAK["bfloat16"] / 1e15}, "kernels": out}),
+          flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--shape", default="tinyllama", choices=sorted(SHAPE_NAMES), help="layer sizes")
+    ap.add_argument("--context", type=int, default=None, help="context length (default: the shape's, 2048 for TinyLlama)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
+    ap.add_argument("--kernels", action="store_true", help="time the dominant kernels alone instead of the engine")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--no-graphs", action="store_true")
@@ -177,8 +301,11 @@ def main() -> int:
     from mini_inference_engine_amd.config import EngineConfig
     from mini_inference_engine_amd.weights import random_tensors
 
-    cfg = tinyllama_config(args.layers)
-    full_layers = 22
+    cfg, full_layers = shape_config(args.shape, args.layers)
+    if args.context is None:
+        args.context = cfg.max_position_embeddings
+    if args.kernels:
+        return measure_kernels(cfg, args)
     dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     elem = 2 if dtype == torch.bfloat16 else 4
     weights = random_tensors(cfg, args.seed, dtype, device="cuda")
@@ -194,6 +321,11 @@ def main() -> int:
         steps = args.steps if b == args.batch else max(10, args.steps // 2)
         dt, captured, ctx = measure_decode(eng, b, args.context, steps, args.warmup, args.seed + b)
         results[b] = dict(tok_s=b * steps / dt, ms=dt / steps * 1e3, captured=captured, steps=steps, context=ctx)
+    short = None
+    if not args.no_points and args.context > 1024:
+        steps = max(10, args.steps // 2)
+        dt, _, ctx = measure_decode(eng, args.batch, 512, steps, args.warmup, args.seed + 7)
+        short = dict(tok_s=args.batch * steps / dt, context=ctx)
     main_r = results[args.batch]
     need = decode_bytes(cfg, args.batch, main_r["context"], elem)
     achieved = need / (main_r["ms"] * 1e-3)
@@ -201,9 +333,10 @@ def main() -> int:
     line = {
         "metric": "decode_tokens_per_second", "value": round(main_r["tok_s"], 1), "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(main_r["ms"], 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": round(main_r["tok_s"] / REFERENCE_B8_TOKENS_PER_S, 2) if args.batch == 8 else None,
+        "scaling": "weak",
+        "vs_baseline": round(main_r["tok_s"] / REFERENCE_B8_TOKENS_PER_S, 2) if args.batch == 8 and args.shape == "tinyllama" else None,
         "dtype": "bf16" if dtype == torch.bfloat16 else "fp32", "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
-        "config": {"model": "TinyLlama-1.1B layer sizes (Llama)", "layers": cfg.num_hidden_layers, "layers_of_config": full_layers,
+        "config": {"model": f"{SHAPE_NAMES[args.shape]} layer sizes (Llama)", "layers": cfg.num_hidden_layers, "layers_of_config": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "global_batch": args.batch, "seq_len": args.context, "context_at_mid_run": main_r["context"],
@@ -214,11 +347,13 @@ def main() -> int:
     }
     if not args.no_points:
         line["points"] = {f"decode_b{b}": round(results[b]["tok_s"], 1) for b in (1, 64)}
+        if short is not None:
+            line["points"][f"decode_b{args.batch}_ctx512"] = round(short["tok_s"], 1)
         t = measure_prefill(eng, 2048 if args.context >= 2048 else args.context, args.seed + 100)
         n = 2048 if args.context >= 2048 else args.context
         line["prefill"] = {"value": round(n / t, 1), "tokens": n, "ms": round(t * 1e3, 3),
                            "frac": round(prefill_flops(cfg, n) / t / FLOP_PEAK[args.dtype], 4)}
-        if cfg.num_hidden_layers == full_layers and args.context >= 1024:
+        if args.shape == "tinyllama" and cfg.num_hidden_layers == full_layers and args.context >= 1024:
             del eng
             torch.cuda.empty_cache()
             mixed = measure_mixed(cfg, weights, dtype, 256, 0, not args.no_graphs)
