@@ -45,6 +45,7 @@ class CacheManager:
         self.released_log: list = []     # (group, page) in release order, kept when keep_log is set
         self.keep_log = False
         self.on_release = None           # callable(group, pages), called as pages go back (debugging)
+        self.on_open = None              # callable(slot), called as a state slot is handed to a request
 
     # ----------------------------------------------------------- lifecycle
     def can_open(self) -> bool:
@@ -58,6 +59,8 @@ class CacheManager:
             raise CacheAccountingError("no state slot free")
         rc = RequestCache(request_id, [[] for _ in self.groups], [0 for _ in self.groups], slot[0])
         self.live[request_id] = rc
+        if self.on_open is not None:
+            self.on_open(slot[0])        # state of fixed size starts afresh with every request
         return rc
 
     def close(self, rc: RequestCache) -> None:

@@ -14,8 +14,6 @@ from dataclasses import dataclass
 
 import torch
 
-from ..parts.base import FixedState, PagedKV
-
 
 @dataclass
 class EntryTensors:
@@ -24,42 +22,42 @@ class EntryTensors:
     v: torch.Tensor | None
     state: torch.Tensor | None
     page_size: int
+    tensors: dict | None = None        # everything the requirement allocated, by name
+    requirement: object = None
 
 
 class CacheStorage:
     def __init__(self, model, page_size: int, pages_per_group: list[int], num_state_slots: int,
                  device, dtype: torch.dtype):
+        """Every cache-owning layer call's requirement allocates its own tensors (parts.base.CacheRequirement);
+        this class only keeps them and knows which belong to which page group."""
         self.page_size = page_size
+        self.device = torch.device(device)
         self.entries: dict[int, EntryTensors] = {}
         for e, ce in model.cache_entries.items():
             r = ce.requirement
-            if isinstance(r, PagedKV):
-                k_shape = (pages_per_group[ce.group], r.num_kv_heads, page_size, r.head_dim)
-                v_shape = (pages_per_group[ce.group], r.num_kv_heads, r.head_dim, page_size)
-                self.entries[e] = EntryTensors(ce.group, torch.zeros(k_shape, dtype=dtype, device=device),
-                                               torch.zeros(v_shape, dtype=dtype, device=device), None, page_size)
-            elif isinstance(r, FixedState):
-                sd = torch.float32 if r.dtype == "float32" else dtype
-                self.entries[e] = EntryTensors(None, None, None, torch.zeros((num_state_slots, *r.shape), dtype=sd,
-                                                                            device=device), page_size)
+            pages = pages_per_group[ce.group] if ce.group is not None else 0
+            t = r.allocate(pages, page_size, num_state_slots, device, dtype)
+            self.entries[e] = EntryTensors(ce.group, t.get("k"), t.get("v"), t.get("state"), page_size, t, r)
 
     def binding(self, entry: int) -> EntryTensors:
         return self.entries[entry]
+
+    def reset_slot(self, slot: int) -> None:
+        """A state slot is handed to a request: every entry with state of fixed size starts it afresh."""
+        for t in self.entries.values():
+            t.requirement.reset_slot(t.tensors, slot)
 
     def poison_pages(self, group: int, pages) -> None:
         """Debugging aid: fill given pages of a group with NaN so a stale read shows."""
         if not pages:
             return
-        idx = torch.tensor(list(pages), dtype=torch.long, device=next(iter(self.entries.values())).k.device)
+        idx = torch.tensor(list(pages), dtype=torch.long, device=self.device)
         for t in self.entries.values():
             if t.group == group:
-                t.k.index_fill_(0, idx, float("nan"))
-                t.v.index_fill_(0, idx, float("nan"))
+                for x in t.tensors.values():
+                    if x.is_floating_point():
+                        x.index_fill_(0, idx, float("nan"))
 
     def num_bytes(self) -> int:
-        n = 0
-        for t in self.entries.values():
-            for x in (t.k, t.v, t.state):
-                if x is not None:
-                    n += x.numel() * x.element_size()
-        return n
+        return sum(x.numel() * x.element_size() for t in self.entries.values() for x in t.tensors.values())

@@ -69,6 +69,12 @@ class LLMEngine:
             print(f"[mini_inference_engine_amd] cache: {self.runner.num_pages} pages x {cfg.block_size} tokens "
                   f"({self.runner.storage.num_bytes() / 2**30:.2f} GiB), weights "
                   f"{self.runner.model.weight_bytes() / 2**30:.2f} GiB, dtype {self.dtype}", flush=True)
+        kept = self.runner.load_report.get("kept_float32", [])
+        if kept:
+            import warnings
+            warnings.warn(f"{len(kept)} weight matrices are stored in float32 and stay so (first: {kept[0]}): their "
+                          f"products run on the 32-bit kernels, much slower than bfloat16; save the checkpoint in "
+                          f"bfloat16 for speed", stacklevel=2)
         self.tokenizer = None
         if load_tokenizer and isinstance(model, str):
             from transformers import AutoTokenizer      # text in and out only; never on the token path

@@ -77,6 +77,8 @@ class ModelRunner:
         self.storage = CacheStorage(self.model, page_size, [self.num_pages] * n_groups, self.num_state_slots,
                                     self.device, self.dtype)
         self.model.attach_cache(self.storage)
+        if any(not ce.requirement.paged for ce in self.model.cache_entries.values()):
+            self.cache.on_open = self.storage.reset_slot
         self.arena = StepArena(max_step_tokens, max_rows, self.max_blocks, n_groups, self.device)
         self.vocab_size = spec.vocab_size
         # The tokens the last step chose, at a fixed address: the next step's rows may take their token

@@ -1,22 +1,29 @@
-"""Continuous batching under a token budget, with recompute preemption.
+"""Which requests run in the next step, and with how many tokens each.
 
-Every step, in this order (inference_engine/scheduler.py:57-102):
- 1. each running request with exactly one token to compute gets it;
- 2. running requests part-way through their prompt get the next portion, as large
-    as the budget allows;
- 3. waiting requests are admitted first come first served, each with as much of
-    its prompt as the budget still allows, unless something was preempted in this
-    very step.
-When a running request cannot get a page, the most recently admitted request is
-preempted: everything it holds goes back, it returns to the front of the queue
-and is later recomputed from its tokens, generated ones included
-(inference_engine/scheduler.py:38-55).  Decided beyond the reference: a request
-that could never fit raises instead of spinning; requests also hold a state slot,
-taken at admission and returned with the pages.
+A step is planned against two resources: the token budget of the step and what the cache manager can still
+hand out (pages per group, state slots).  The plan is built in three stages, in the order that fixes who
+wins when a resource runs short (the behaviour of inference_engine/scheduler.py:57-102):
+
+ 1. requests that are running and need exactly one token (they are decoding) get it;
+ 2. requests that are running and still have part of their prompt to run get the next portion, as large
+    as the budget leaves;
+ 3. waiting requests are admitted first come first served, each with as much of its prompt as the budget
+    leaves, unless the step had to evict somebody: then it admits nobody.
+
+Rules of this engine beside those stages:
+  * a request whose last token is already on its way (``Sequence.ending``) asks for nothing more;
+  * admission takes a state slot as well as pages, and keeps a small share of the pages free for the
+    requests already running (not when nothing runs: a request alone may use the last page);
+  * when a running request cannot get a page, the request admitted last gives back everything it holds and
+    goes to the front of the queue, to be run again from its tokens (inference_engine/scheduler.py:38-55);
+    it also leaves the plan of the step if it was in it;
+  * what can never run (longer than the cache holds for one request, or stuck at the head of the queue with
+    nothing running) raises ``RequestTooLarge`` instead of planning empty steps for ever.
 """
 from __future__ import annotations
 
 from collections import deque
+from dataclasses import dataclass, field
 
 from ..cache import CacheManager
 from ..config.engine_config import EngineConfig
@@ -27,107 +34,130 @@ class RequestTooLarge(RuntimeError):
     pass
 
 
+@dataclass
+class _Plan:
+    """A step being planned: the tokens still to give away and who got how many so far."""
+    budget: int
+    single: list = field(default_factory=list)       # (request, 1): one row each, first in the step
+    portions: list = field(default_factory=list)     # (request, n > 1, or the one token of a prompt of one)
+    evicted: bool = False
+
+    def give(self, seq: Sequence, n: int, portion: bool) -> None:
+        (self.portions if portion else self.single).append((seq, n))
+        self.budget -= n
+
+    def drop(self, seq: Sequence) -> None:
+        """``seq`` was evicted after it had been given tokens: they go back to the budget."""
+        for rows in (self.single, self.portions):
+            for entry in [e for e in rows if e[0] is seq]:
+                rows.remove(entry)
+                self.budget += entry[1]
+
+    def rows(self) -> list:
+        return self.single + self.portions
+
+
 class Scheduler:
     def __init__(self, cfg: EngineConfig, cache: CacheManager):
         self.cfg = cfg
         self.cache = cache
         self.waiting: deque[Sequence] = deque()
-        self.running: list[Sequence] = []
+        self.running: list[Sequence] = []            # in order of admission: the last is the first to be evicted
         self.num_preemptions = 0
-        # keep about 1% of the pages free at admission so running requests can grow
-        self.watermark = max(1, min(cache.usable_pages(g) for g in range(len(cache.groups))) // 100) \
-            if cache.groups else 0
+        # the share of the pages admission leaves to the running requests: about one in a hundred
+        groups = range(len(cache.groups))
+        self.watermark = max(1, min(cache.usable_pages(g) for g in groups) // 100) if cache.groups else 0
 
+    # ------------------------------------------------------------------ queue
     def add(self, seq: Sequence) -> None:
-        limit = self.cache.max_tokens_one_request()
-        worst = min(seq.prompt_len + seq.params.max_tokens, self.cfg.max_model_len)
-        if seq.prompt_len > limit or worst > limit:
+        room = self.cache.max_tokens_one_request()
+        longest = min(seq.prompt_len + seq.params.max_tokens, self.cfg.max_model_len)
+        if max(seq.prompt_len, longest) > room:
             raise RequestTooLarge(
                 f"request of {seq.prompt_len} prompt + {seq.params.max_tokens} new tokens can never fit: "
-                f"the cache holds {limit} tokens for one request")
+                f"the cache holds {room} tokens for one request")
         self.waiting.append(seq)
 
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
 
-    # ------------------------------------------------------------ preemption
-    def _preempt(self, seq: Sequence) -> None:
-        self.running.remove(seq)
-        self.cache.close(seq.cache)
-        seq.cache = None
-        seq.num_computed = 0
-        seq.status = Status.WAITING
-        seq.num_preemptions += 1
-        self.num_preemptions += 1
-        self.waiting.appendleft(seq)
+    # ------------------------------------------------------------------- rules
+    def _portion(self, seq: Sequence, budget: int) -> int:
+        """Tokens of ``seq`` that may run under ``budget``; 0: not in this step."""
+        want = seq.num_new_tokens
+        if seq.ending or want <= 0 or budget <= 0:
+            return 0
+        if want <= budget:
+            return want
+        return budget if self.cfg.enable_chunked_prefill else 0
 
-    def _reserve_or_preempt(self, seq: Sequence, n: int) -> bool:
-        """False if ``seq`` itself had to go."""
+    def _evict(self, plan: _Plan) -> Sequence:
+        """The request admitted last gives everything back and will be run again from its tokens."""
+        victim = self.running.pop()
+        self.cache.close(victim.cache)
+        victim.cache = None
+        victim.num_computed = 0
+        victim.status = Status.WAITING
+        victim.num_preemptions += 1
+        self.num_preemptions += 1
+        self.waiting.appendleft(victim)
+        plan.drop(victim)
+        plan.evicted = True
+        return victim
+
+    def _grant(self, seq: Sequence, n: int, plan: _Plan, portion: bool) -> None:
+        """Pages for ``n`` more tokens of a running request, evicting from the end of the line until they are
+        there; if the line ends at ``seq`` itself it goes too, and gets nothing."""
         while not self.cache.reserve(seq.cache, seq.num_computed, n):
-            victim = self.running[-1]
-            if victim is seq and len(self.running) == 1:
-                raise RequestTooLarge(
-                    f"request {seq.seq_id} alone cannot get pages for {seq.num_computed + n} tokens")
-            self._preempt(victim)
-            if victim is seq:
-                return False
+            if self.running[-1] is seq and len(self.running) == 1:
+                raise RequestTooLarge(f"request {seq.seq_id} alone cannot get pages for {seq.num_computed + n} tokens")
+            if self._evict(plan) is seq:
+                return
+        plan.give(seq, n, portion)
+
+    def _admit(self, seq: Sequence, n: int, plan: _Plan) -> bool:
+        """A state slot and the pages of its first ``n`` tokens, or nothing."""
+        if not self.cache.can_open():
+            return False
+        held = self.cache.open(seq.seq_id)
+        keep_free = self.watermark if self.running else 0
+        if not self.cache.reserve(held, 0, n, watermark=keep_free):
+            self.cache.close(held)
+            return False
+        seq.cache = held
+        seq.status = Status.RUNNING
+        self.running.append(seq)
+        plan.give(seq, n, portion=True)
         return True
 
-    # -------------------------------------------------------------- one step
+    # ---------------------------------------------------------------- one step
     def schedule(self) -> list[tuple[Sequence, int]]:
-        budget = self.cfg.max_num_batched_tokens
-        decodes, prefills = [], []
-        preemptions_before = self.num_preemptions
-
-        for seq in list(self.running):
-            if seq.status is not Status.RUNNING or seq.num_new_tokens != 1 or seq.ending:
-                continue
-            if budget == 0:
+        plan = _Plan(self.cfg.max_num_batched_tokens)
+        # stages 1 and 2 walk the line as it stood when the step began; who is evicted on the way is skipped
+        line = list(self.running)
+        for decoding in (True, False):
+            for seq in line:
+                if seq.status is not Status.RUNNING or (seq.num_new_tokens == 1) != decoding:
+                    continue
+                n = self._portion(seq, plan.budget)
+                if n:
+                    self._grant(seq, n, plan, portion=not decoding)
+        # stage 3
+        while self.waiting and not plan.evicted and len(self.running) < self.cfg.max_num_seqs:
+            head = self.waiting[0]
+            n = self._portion(head, plan.budget)
+            if not n or not self._admit(head, n, plan):
                 break
-            if self._reserve_or_preempt(seq, 1):
-                decodes.append((seq, 1))
-                budget -= 1
-
-        for seq in list(self.running):
-            if seq.status is not Status.RUNNING or seq.num_new_tokens <= 1 or budget == 0 or seq.ending:
-                continue
-            n = min(seq.num_new_tokens, budget)
-            if not self.cfg.enable_chunked_prefill and n < seq.num_new_tokens:
-                continue
-            if self._reserve_or_preempt(seq, n):
-                prefills.append((seq, n))
-                budget -= n
-
-        # a request scheduled above may have been preempted to make room afterwards
-        decodes = [(s, n) for s, n in decodes if s.status is Status.RUNNING]
-        prefills = [(s, n) for s, n in prefills if s.status is Status.RUNNING]
-
-        preempted_now = self.num_preemptions != preemptions_before
-        while (self.waiting and budget > 0 and len(self.running) < self.cfg.max_num_seqs and not preempted_now
-               and self.cache.can_open()):
-            seq = self.waiting[0]
-            n = min(seq.num_new_tokens, budget)
-            if not self.cfg.enable_chunked_prefill and n < seq.num_new_tokens:
-                break
-            rc = self.cache.open(seq.seq_id)
-            # alone, a request may use the last pages: nothing else is there to grow
-            mark = self.watermark if self.running else 0
-            if not self.cache.reserve(rc, 0, n, watermark=mark):
-                self.cache.close(rc)
-                break
-            seq.cache = rc
             self.waiting.popleft()
-            seq.status = Status.RUNNING
-            self.running.append(seq)
-            prefills.append((seq, n))
-            budget -= n
 
-        if not decodes and not prefills and self.has_work() and not any(s.ending for s in self.running):
+        rows = plan.rows()
+        if not rows and self.has_work() and not any(s.ending for s in self.running):
             # (a request whose last token is on its way will make room when it ends)
             raise RequestTooLarge("nothing can be scheduled although requests are waiting: "
                                   "the head of the queue does not fit the cache or the budget")
-        return decodes + prefills
+        return rows
 
+    # ------------------------------------------------------------- after a step
     def advance(self, seq: Sequence, n: int) -> None:
         """``n`` more tokens of ``seq`` are in the cache."""
         seq.num_computed += n

@@ -93,6 +93,19 @@ def _build_dirs() -> list[str]:
     return dirs
 
 
+def _trusted(d: str) -> bool:
+    """Libraries are loaded into the process, so a folder outside the package counts only if it is this
+    user's own and nobody else can write to it (the per-user folder under the temporary directory has a
+    name anyone could have created first)."""
+    if os.path.dirname(os.path.abspath(d)) == os.path.abspath(CSRC):
+        return True
+    try:
+        st = os.stat(d)
+    except OSError:
+        return False
+    return (not hasattr(os, "getuid") or st.st_uid == os.getuid()) and not (st.st_mode & 0o022)
+
+
 def library_file(module: str, defines: tuple = ()) -> str:
     return f"{module}{_tag(defines)}-{_digest(module, defines)}.so"
 
@@ -101,7 +114,7 @@ def find_built(module: str, defines: tuple = ()) -> str | None:
     name = library_file(module, defines)
     for d in _build_dirs():
         p = os.path.join(d, name)
-        if os.path.isfile(p):
+        if os.path.isfile(p) and _trusted(d):
             return p
     return None
 
@@ -123,7 +136,9 @@ def build(module: str, defines: tuple = (), verbose: bool = True) -> str:
     out_dir = None
     for d in _build_dirs():
         try:
-            os.makedirs(d, exist_ok=True)
+            os.makedirs(d, mode=0o700, exist_ok=True)
+            if not _trusted(d):
+                continue
             fd, probe = tempfile.mkstemp(dir=d, prefix=".w")
             os.close(fd)
             os.remove(probe)

@@ -6,7 +6,7 @@ between architectures is the DecoderSpec their builder returns.
 """
 from __future__ import annotations
 
-from ..parts.base import CacheBinding, DecoderSpec, FixedState, PagedKV, ParamSpec, Part
+from ..parts.base import CacheBinding, CacheRequirement, DecoderSpec, ParamSpec, Part
 
 
 class CacheEntry:
@@ -15,7 +15,7 @@ class CacheEntry:
     def __init__(self, entry: int, requirement):
         self.entry = entry
         self.requirement = requirement
-        self.group = None       # page group id for PagedKV
+        self.group = None       # page group id, for requirements that keep data in pages
 
 
 class Decoder:
@@ -27,19 +27,22 @@ class Decoder:
         # cache needs, one per owning run-order entry; groups by window
         self.cache_entries: dict[int, CacheEntry] = {}
         self.page_groups: list = []       # window (None = all keys) of each page group
+        group_keys: list = []
         for e, call in enumerate(spec.schedule):
             if call.cache_of is not None:
                 continue
             req = spec.layers[call.layer].mixer.cache_requirement()
             if req is None:
                 continue
+            if not isinstance(req, CacheRequirement):
+                raise TypeError(f"cache_requirement() of layer {call.layer} returned {req!r}, not a CacheRequirement")
             ce = CacheEntry(e, req)
-            if isinstance(req, PagedKV):
-                if req.window not in self.page_groups:
+            if req.paged:
+                key = req.page_group_key()
+                if key not in group_keys:
+                    group_keys.append(key)
                     self.page_groups.append(req.window)
-                ce.group = self.page_groups.index(req.window)
-            elif not isinstance(req, FixedState):
-                raise TypeError(f"unknown cache requirement {req!r}")
+                ce.group = group_keys.index(key)
             self.cache_entries[e] = ce
         self.bindings: list[CacheBinding] = []
 
@@ -81,8 +84,7 @@ class Decoder:
         out = [0] * len(self.page_groups)
         for ce in self.cache_entries.values():
             if ce.group is not None:
-                r = ce.requirement
-                out[ce.group] += 2 * page_size * r.num_kv_heads * r.head_dim * element_size
+                out[ce.group] += ce.requirement.bytes_per_page(page_size, element_size)
         return out
 
     def attach_cache(self, storage) -> None:
@@ -96,7 +98,8 @@ class Decoder:
                 continue
             b = storage.binding(owner)
             self.bindings.append(CacheBinding(group=b.group, k=b.k, v=b.v, state=b.state,
-                                              read_only=call.cache_of is not None, page_size=b.page_size))
+                                              read_only=call.cache_of is not None, page_size=b.page_size,
+                                              tensors=b.tensors))
 
     # -------------------------------------------------------------- forward
     def forward(self, step):

@@ -1,5 +1,5 @@
 from .attention import Attention
-from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Block, CacheBinding, DecoderSpec,
+from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Block, CacheBinding, CacheRequirement, DecoderSpec,
                    FeedForward, FixedState, LayerCall, Mixer, Norm, PagedKV, ParamSpec, Part, PositionEncoding,
                    Source, register_block, register_feed_forward, register_mixer, register_norm,
                    register_position_encoding)

@@ -49,11 +49,12 @@ class ParamSpec:
     shape: tuple
     sources: tuple
     integer: bool = False   # integer tables are kept as int32
+    init: str = "weight"    # how the random-weights mode draws it: "weight" N(0, std), "scale" 1 + N(0, std), "zeros"
 
     @staticmethod
-    def single(attr: str, name: str, shape: Sequence[int], integer: bool = False) -> "ParamSpec":
+    def single(attr: str, name: str, shape: Sequence[int], integer: bool = False, init: str = "weight") -> "ParamSpec":
         shape = tuple(int(s) for s in shape)
-        return ParamSpec(attr, shape, (Source(name, shape, 0),), integer)
+        return ParamSpec(attr, shape, (Source(name, shape, 0),), integer, init)
 
     @staticmethod
     def stacked(attr: str, pieces: Sequence[tuple]) -> "ParamSpec":
@@ -97,20 +98,69 @@ class Part:
 
 
 # ---------------------------------------------------------------- cache needs
+class CacheRequirement:
+    """What a mixer call wants kept between steps.  The model, the cache manager and the storage know no
+    kind by name: they ask the requirement.  A new kind (another layout per token, a latent instead of
+    keys and values, several state tensors) is a subclass; nothing else changes.
+
+    paged        True: data per token, in pages that the cache manager hands out per request; requirements
+                 with equal ``page_group_key()`` share page ids and block tables.
+    window       for paged data: how many keys back a query looks at most (None = all); pages that lie
+                 wholly before the window are given back.
+    bytes_per_page(page_size, element_size)   what one page id costs in this entry (sizes the pool)
+    allocate(num_pages, page_size, num_slots, device, act_dtype) -> dict of tensors, handed to the mixer as
+                 CacheBinding.k / .v / .state (keys of those names) and CacheBinding.tensors (all of them)
+    reset_slot(tensors, slot)   state of fixed size: called when a slot is handed to a request
+    """
+    paged = False
+    window = None
+
+    def page_group_key(self):
+        return self.window
+
+    def bytes_per_page(self, page_size: int, element_size: int) -> int:
+        return 0
+
+    def allocate(self, num_pages: int, page_size: int, num_slots: int, device, act_dtype) -> dict:
+        raise NotImplementedError
+
+    def reset_slot(self, tensors: dict, slot: int) -> None:
+        pass
+
+
 @dataclass(frozen=True)
-class PagedKV:
-    """Keys and values of every token in pages; ``window`` keys back at most, or all."""
+class PagedKV(CacheRequirement):
+    """Keys and values of every token in pages; ``window`` keys back at most, or all.  Keys
+    [pages, kv_heads, page, head_dim]; values [pages, kv_heads, head_dim, page] (a page's values transposed:
+    both are then what the attention kernels' matrix instructions take straight from memory)."""
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    paged = True
+
+    def bytes_per_page(self, page_size, element_size):
+        return 2 * page_size * self.num_kv_heads * self.head_dim * element_size
+
+    def allocate(self, num_pages, page_size, num_slots, device, act_dtype):
+        import torch
+        return {"k": torch.zeros((num_pages, self.num_kv_heads, page_size, self.head_dim), dtype=act_dtype, device=device),
+                "v": torch.zeros((num_pages, self.num_kv_heads, self.head_dim, page_size), dtype=act_dtype, device=device)}
 
 
 @dataclass(frozen=True)
-class FixedState:
-    """Per-request state of fixed size, indexed by the request's state slot.
-    ``dtype``: 'float32' or 'activation'."""
+class FixedState(CacheRequirement):
+    """Per-request state of fixed size, [slots, *shape], indexed by the request's state slot; zeroed when
+    the slot is handed to a request.  ``dtype``: 'float32' or 'activation'."""
     shape: tuple
     dtype: str = "float32"
+
+    def allocate(self, num_pages, page_size, num_slots, device, act_dtype):
+        import torch
+        dt = torch.float32 if self.dtype == "float32" else act_dtype
+        return {"state": torch.zeros((num_slots, *self.shape), dtype=dt, device=device)}
+
+    def reset_slot(self, tensors, slot):
+        tensors["state"][slot].zero_()
 
 
 @dataclass
@@ -122,6 +172,7 @@ class CacheBinding:
     state: Any = None                 # [slots, *shape]
     read_only: bool = False           # entry belongs to another layer call
     page_size: int = 0
+    tensors: Any = None               # everything the requirement allocated, by name
 
 
 class Norm(Part):

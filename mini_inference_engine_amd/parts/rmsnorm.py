@@ -20,7 +20,7 @@ class RMSNorm(Norm):
         self.weight = None
 
     def params(self):
-        return [ParamSpec.single("weight", self.weight_name, (self.width,))]
+        return [ParamSpec.single("weight", self.weight_name, (self.width,), init="scale")]
 
     def lazy(self, x, residual, rows=None):
         if isinstance(x, Normed):

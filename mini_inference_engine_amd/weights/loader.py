@@ -128,14 +128,19 @@ def load_weights(model, source, device, mode: torch.dtype) -> dict:
         raise WeightError(source.folder, missing, unexpected, wrong)
 
     ignored = sorted(n for n in present if n not in wanted)
+    kept_float32 = []
     for part, spec in specs:
         pieces = [source.tensor(s.name) for s in spec.sources]
         kinds = {storage_dtype(t.dtype, mode, spec.integer) for t in pieces}
         dtype = torch.float32 if torch.float32 in kinds else kinds.pop()
+        if dtype == torch.float32 and mode != torch.float32 and len(spec.shape) >= 2:
+            # kept as stored; the products of this matrix then run on the 32-bit kernels, far slower than the
+            # bfloat16 ones: worth a line, since a checkpoint saved in float32 does this to every layer
+            kept_float32 += [s.name for s, t in zip(spec.sources, pieces) if t.dtype in (torch.float32, torch.float64)]
         buf = torch.empty(spec.shape, dtype=dtype, device=device)
         for s, t in zip(spec.sources, pieces):
             rows = s.shape[0] if s.shape else 1
             dst = buf[s.row_offset:s.row_offset + rows] if len(spec.sources) > 1 else buf
             dst.copy_(t.to(dtype))
         part.bind(spec.attr, buf)
-    return {"tensors": len(wanted), "ignored": ignored}
+    return {"tensors": len(wanted), "ignored": ignored, "kept_float32": kept_float32}

@@ -30,9 +30,15 @@ def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std: 
                 continue
             if spec.integer:
                 raise NotImplementedError("random integer tables")
+            # every tensor draws from the generator, whatever its kind, so that adding a part does not shift
+            # the values of the parts after it
             t = torch.randn(s.shape, generator=gen, dtype=torch.float32, device=device) * std
-            if len(s.shape) == 1:
+            if spec.init == "scale":
                 t = t + 1.0
+            elif spec.init == "zeros":
+                t = torch.zeros_like(t)
+            elif spec.init != "weight":
+                raise ValueError(f"{s.name}: unknown init {spec.init!r} (weight, scale or zeros)")
             out[s.name] = t.to(dtype).contiguous()
     return out
 

@@ -190,3 +190,22 @@ def test_no_safetensors_and_sharded_folders(tmp_path):
     model = build(TINY_A)
     load_weights(model, str(tmp_path), "cpu", torch.float32)
     assert torch.equal(model.spec.embedding.weight, w["model.embed_tokens.weight"])
+
+
+def test_float32_matrices_in_bfloat16_mode_are_reported(tiny_models):
+    """A tensor stored in 32-bit stays so; for a matrix that means the slow 32-bit products, so the load
+    report names it (and the entry point warns)."""
+    from mini_inference_engine_amd.models.decoder import Decoder
+    from mini_inference_engine_amd.config.registry import architecture_of
+    from mini_inference_engine_amd.weights import load_weights
+    m = tiny_models["A"]
+    mixed = dict(m["weights_bf16"])
+    mixed["model.layers.1.mlp.down_proj.weight"] = m["weights"]["model.layers.1.mlp.down_proj.weight"]      # float32
+    mixed["model.norm.weight"] = m["weights"]["model.norm.weight"]                                          # a vector
+    model = Decoder(architecture_of(m["config"]).build(m["config"]))
+    report = load_weights(model, mixed, "cpu", torch.bfloat16)
+    assert report["kept_float32"] == ["model.layers.1.mlp.down_proj.weight"], "matrices only; vectors are cheap"
+    assert model.spec.layers[1].feed_forward.w_down.dtype == torch.float32
+    assert model.spec.layers[0].feed_forward.w_down.dtype == torch.bfloat16
+    report = load_weights(Decoder(architecture_of(m["config"]).build(m["config"])), m["weights_bf16"], "cpu", torch.bfloat16)
+    assert report["kept_float32"] == []

@@ -24,7 +24,7 @@ from torch_backend import TorchBackend
 
 from mini_inference_engine_amd.config import ModelConfig, register_architecture, unregister_architecture
 from mini_inference_engine_amd.engine.runner import ModelRunner
-from mini_inference_engine_amd.parts import (Attention, DecoderSpec, Embedding, FeedForward, FixedState, LayerCall,
+from mini_inference_engine_amd.parts import (Attention, CacheRequirement, DecoderSpec, Embedding, FeedForward, FixedState, LayerCall,
                                              LMHead, Mixer, ParamSpec, PositionEncoding, PreNormBlock, RMSNorm,
                                              RotaryHalfSplit, SwiGLU, register_feed_forward, register_mixer,
                                              register_position_encoding)
@@ -35,9 +35,27 @@ from mini_inference_engine_amd.weights import random_tensors
 WIDTH, HEADS, KV, HD, INTER, VOCAB, WINDOW, DECAY = 48, 3, 1, 16, 80, 97, 8, 0.8
 
 
+class DecayState(CacheRequirement):
+    """A cache kind of this file's own: the running sum of a request, and how many tokens went into it.
+    The engine allocates it, hands it to the mixer, and starts a slot afresh when a request gets it."""
+
+    def __init__(self, width):
+        self.width = width
+
+    def allocate(self, num_pages, page_size, num_slots, device, act_dtype):
+        return {"state": torch.zeros((num_slots, self.width), dtype=torch.float32, device=device),
+                "fed": torch.zeros(num_slots, dtype=torch.int64, device=device)}
+
+    def reset_slot(self, tensors, slot):
+        tensors["state"][slot].zero_()
+        tensors["fed"][slot] = 0
+
+
 @register_mixer("toy_decay")
 class DecayMixer(Mixer):
-    """s_t = decay * s_{t-1} + x_t per request, y_t = s_t W^T.  The state lives in the request's slot."""
+    """s_t = decay * s_{t-1} + x_t per request, y_t = s_t W^T.  The state lives in the request's slot; it is
+    never reset here: the cache hands out slots that start at zero.  On the GPU the scan is a kernel of this
+    test's own (tests/toy_decay.hip), registered with the engine's loader in tests/toy_kernels.py."""
 
     def __init__(self, width, decay, prefix):
         self.width, self.decay, self.prefix = width, decay, prefix
@@ -47,19 +65,32 @@ class DecayMixer(Mixer):
         return [ParamSpec.single("weight", f"{self.prefix}.weight", (self.width, self.width))]
 
     def cache_requirement(self):
-        return FixedState((self.width,), "float32")
+        return DecayState(self.width)
 
     def forward(self, x, step, cache, add_to=None):
-        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
         starts, first_pos, slots = step.host["row_start"], step.host["row_position"], step.host["state_slots"]
+        fed = cache.tensors["fed"]
         for r in range(step.num_rows):
-            a, b = int(starts[r]), int(starts[r + 1])
-            slot = int(slots[r])
-            s = cache.state[slot].clone() if first_pos[r] > 0 else torch.zeros_like(cache.state[slot])
-            for t in range(a, b):
-                s = self.decay * s + x[t].float()
-                out[t] = s
-            cache.state[slot] = s
+            if int(slots[r]) != 0:           # (slot 0 is the scratch slot of padding rows)
+                assert int(fed[int(slots[r])]) == int(first_pos[r]), "the slot's state is not this request's so far"
+                fed[int(slots[r])] += int(starts[r + 1] - starts[r])
+        xf = x.float().contiguous()
+        out = torch.empty_like(xf)
+        if x.device.type == "cuda":
+            import toy_kernels  # noqa: F401  (registers the module)
+            from mini_inference_engine_amd.kernels import library
+            lib = self.ops.lib("toy_decay")
+            library.check(lib, lib.toy_decay_scan(xf.data_ptr(), out.data_ptr(), cache.state.data_ptr(),
+                                                  step.row_start.data_ptr(), step.state_slots.data_ptr(), step.num_rows,
+                                                  self.width, self.decay, torch.cuda.current_stream().cuda_stream))
+        else:
+            for r in range(step.num_rows):
+                slot = int(slots[r])
+                s = cache.state[slot].clone()
+                for t in range(int(starts[r]), int(starts[r + 1])):
+                    s = self.decay * s + xf[t]
+                    out[t] = s
+                cache.state[slot] = s
         return self.ops.linear(out.to(x.dtype), self.weight)
 
 
@@ -67,16 +98,18 @@ class DecayMixer(Mixer):
 class TanhGate(FeedForward):
     def __init__(self, width, inner, prefix):
         self.width, self.inner, self.prefix = width, inner, prefix
-        self.w_in = self.w_out = None
+        self.w_in = self.w_out = self.bias = None
 
     def params(self):
         return [ParamSpec.stacked("w_in", [(f"{self.prefix}.a.weight", (self.inner, self.width)),
                                            (f"{self.prefix}.b.weight", (self.inner, self.width))]),
-                ParamSpec.single("w_out", f"{self.prefix}.out.weight", (self.width, self.inner))]
+                ParamSpec.single("w_out", f"{self.prefix}.out.weight", (self.width, self.inner)),
+                # a tensor of one dimension that is no norm weight: the random-weights mode must not centre it at 1
+                ParamSpec.single("bias", f"{self.prefix}.a.bias", (self.inner,), init="zeros")]
 
     def forward(self, x, step, add_to=None):
         ab = self.ops.linear(x, self.w_in).float()
-        h = torch.tanh(ab[:, :self.inner]) * ab[:, self.inner:]
+        h = torch.tanh(ab[:, :self.inner] + self.bias.float()) * ab[:, self.inner:]
         return self.ops.linear(h.to(x.dtype), self.w_out, add_to=add_to)
 
 
@@ -124,6 +157,9 @@ def toy():
     # layer to layer; q and k doubled: scores with a standard deviation of about 4, far from uniform, so
     # which keys are seen matters, yet not so sharp that the rounding of a score shows in the probabilities
     weights = random_tensors(cfg, 9, torch.float32, std=WIDTH ** -0.5)
+    assert float(weights["l0.ff.a.bias"].abs().max()) == 0.0 and abs(float(weights["l0.n1"].mean()) - 1.0) < 0.1, \
+        "the random-weights mode draws each tensor as its part declares it"
+    weights["l0.ff.a.bias"] = torch.linspace(-0.5, 0.5, 40)          # (so that the bias matters to the result)
     for k in weights:
         if k.endswith("q_proj.weight") or k.endswith("k_proj.weight"):
             weights[k] = weights[k] * 2
@@ -163,7 +199,7 @@ def plain_toy(weights, ids):
         ys.append(state)
     s = s + torch.stack(ys) @ w["l0.mix.weight"].T
     x = plain.rms_norm(s, w["l0.n2"], 1e-5)
-    s = s + (torch.tanh(x @ w["l0.ff.a.weight"].T) * (x @ w["l0.ff.b.weight"].T)) @ w["l0.ff.out.weight"].T
+    s = s + (torch.tanh(x @ w["l0.ff.a.weight"].T + w["l0.ff.a.bias"]) * (x @ w["l0.ff.b.weight"].T)) @ w["l0.ff.out.weight"].T
     s, _ = attention_layer(s, 1, window=WINDOW)
     s, kv2 = attention_layer(s, 2)
     s, _ = attention_layer(s, 1, window=WINDOW)
@@ -197,6 +233,22 @@ def run_family(toy, family, tmp_path, device, dtype, backend, tol, plain_model=N
         # the windowed group handed pages back while requests were still running
         assert [p for g, p in runner.cache.released_log if g == 0], "windowed pages must be released"
     return runner, worst
+
+
+def test_a_state_slot_starts_afresh_with_every_request(toy):
+    """The cache resets what a slot holds when it hands the slot out (the requirement says how): the toy
+    mixer never looks at a row's position to decide whether to start from zero."""
+    cfg, weights = toy
+    runner = ModelRunner(cfg, weights=weights, dtype="float32", device="cpu", backend=TorchBackend(torch.float32),
+                         num_pages=8, max_rows=4, max_step_tokens=64)
+    entry = next(t for t in runner.storage.entries.values() if t.state is not None)
+    entry.tensors["state"].fill_(7.0)
+    entry.tensors["fed"].fill_(99)
+    rc = runner.cache.open("a")
+    assert float(entry.tensors["state"][rc.state_slot].abs().max()) == 0.0 and int(entry.tensors["fed"][rc.state_slot]) == 0
+    other = [s for s in range(1, runner.num_state_slots) if s != rc.state_slot][0]
+    assert float(entry.tensors["state"][other].min()) == 7.0, "only the slot handed out is reset"
+    runner.cache.close(rc)
 
 
 @pytest.mark.parametrize("family", ["whole", "decode_tail", "portions", "mixed"])

@@ -53,6 +53,25 @@ def test_rotation_is_complex_multiplication_on_half_split_pairs():
     torch.testing.assert_close((y[..., :D // 2] ** 2 + y[..., D // 2:] ** 2), (x[..., :D // 2] ** 2 + x[..., D // 2:] ** 2))
 
 
+def test_rotation_frequencies_are_a_geometric_ladder_from_one_down():
+    """What fixes the frequency schedule without re-typing its expression: pair 0 turns by one radian a
+    position (at position p its angle is p), every next pair turns slower by the same factor, and that factor
+    is such that a pair numbered D / 2, one past the last, would turn theta times slower than pair 0
+    (inference_engine/model.py:56-58 there: the exponents are 0, 2/D, ..., (D - 2)/D of theta).  A ladder over
+    D / 2 - 1 steps (exponent j / (D/2 - 1)), one that starts a step late (pair 0 slower than a radian), or
+    exponents j / D, fail one of these."""
+    for theta, D in ((10000.0, 64), (500000.0, 32), (1000.0, 48)):
+        cos, sin = plain.rope_table(theta, D, 8)
+        angle = torch.atan2(sin[1, :D // 2].double(), cos[1, :D // 2].double())      # position 1: below pi for all pairs
+        assert abs(float(angle[0]) - 1.0) < 1e-6
+        ratio = angle[1:] / angle[:-1]
+        torch.testing.assert_close(ratio, ratio[0].expand_as(ratio), atol=0, rtol=1e-5)
+        assert abs(float(ratio[0]) ** (D // 2) * theta - 1.0) < 1e-4
+        # the table's two halves are the same angles (the pair (j, j + D / 2) turns together), and row p is p times row 1
+        torch.testing.assert_close(cos[:, :D // 2], cos[:, D // 2:])
+        torch.testing.assert_close(torch.cos(5 * angle).float(), cos[5, :D // 2], atol=1e-5, rtol=0)
+
+
 def test_rotated_scores_depend_on_distance_only():
     D = 32
     cos, sin = (t.double() for t in plain.rope_table(500000.0, D, 200))
@@ -76,6 +95,11 @@ def test_attention_is_the_library_routine(H, Hkv):
     lib = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1).repeat_interleave(g, 0)[None],
                                          v.transpose(0, 1).repeat_interleave(g, 0)[None], is_causal=True, scale=0.3)
     torch.testing.assert_close(out, lib[0].transpose(0, 1))
+    # the scale the model uses, 1 / sqrt(head size), is the library routine's own default (the reference calls it
+    # with that value, inference_engine/model.py:151-152 there); plain.attention_block passes exactly this
+    lib = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1).repeat_interleave(g, 0)[None],
+                                         v.transpose(0, 1).repeat_interleave(g, 0)[None], is_causal=True)
+    torch.testing.assert_close(plain.causal_attention(q, k, v, 1.0 / math.sqrt(D)), lib[0].transpose(0, 1))
     torch.testing.assert_close(out[0], v[0].repeat_interleave(g, 0))        # one key: the output is its value
     if Hkv > 1 and g > 1:
         tiled = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1).repeat(g, 1, 1)[None],
