@@ -153,9 +153,11 @@ class HipBackend(KernelBackend):
         if sink is not None and sink.norm_weight is not None:
             g = sink.norm_weight
             tiles = -(-n_out // 16)
-            made = {"x": torch.empty((M, n_out), dtype=torch.bfloat16, device=w.device),
+            # rows 64 bytes apart from a multiple of 4 KB: rows that are exactly 4 KB long fall on the same cache
+            # channels when every workgroup reads all of them at once (qkv and o products 0.4 us faster at 8 rows)
+            made = {"x": torch.empty((M, n_out + 32), dtype=torch.bfloat16, device=w.device)[:, :n_out],
                     "ss": torch.empty((M, (tiles + 3) // 4 * 4), dtype=torch.float32, device=w.device), "tiles": tiles}
-            norm_args = [_ptr(g), int(g.dtype == torch.float32), _ptr(made["x"]), n_out, _ptr(made["ss"]), None, 0,
+            norm_args = [_ptr(g), int(g.dtype == torch.float32), _ptr(made["x"]), made["x"].stride(0), _ptr(made["ss"]), None, 0,
                          0.0, None]
         elif prepared is not None:
             norm_args = [None, 0, None, 0, None, _ptr(prepared["ss"]), prepared["tiles"], float(eps), _ptr(rows)]
