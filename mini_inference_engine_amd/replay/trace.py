@@ -89,7 +89,9 @@ def main(argv=None) -> int:
     args = _parser().parse_args(argv)
     from ..engine.runner import ModelRunner
     page = args.block_size
-    pages = -(-args.max_tokens // page) + 1          # + the scratch page
+    # --max-tokens counts every live request rounded up to 64 tokens, so whole pages cover it; a page more for each
+    # of the four requests that may be live keeps a count that was not rounded from running out, + the scratch page
+    pages = -(-args.max_tokens // page) + 4 + 1
     runner = ModelRunner(args.model, dtype=args.dtype, device=args.device, page_size=page, num_pages=pages,
                          max_step_tokens=max(64, args.max_tokens), max_rows=64)
     if args.hip_graphs:

@@ -38,7 +38,13 @@ TINY_C = dict(architectures=["LlamaForCausalLM"], vocab_size=331, hidden_size=12
               num_hidden_layers=2, num_attention_heads=5, num_key_value_heads=5, head_dim=48,
               rms_norm_eps=1e-5, rope_theta=1000.0, max_position_embeddings=512, tie_word_embeddings=False,
               eos_token_id=1)
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 5)}
+# A fourth with sizes the vector paths of the kernels do not like: a width and a feed-forward size that are no
+# multiple of 8 (bfloat16 rows are then not 16-byte aligned), an odd vocabulary, heads wider than the width / heads.
+TINY_D = dict(architectures=["LlamaForCausalLM"], vocab_size=301, hidden_size=70, intermediate_size=177,
+              num_hidden_layers=2, num_attention_heads=3, num_key_value_heads=3, head_dim=32,
+              rms_norm_eps=1e-4, rope_theta=5000.0, max_position_embeddings=160, tie_word_embeddings=True,
+              eos_token_id=300)
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 5), "D": (TINY_D, 8)}
 
 
 @pytest.fixture(scope="session")

@@ -24,7 +24,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 F32_TOL = 2e-5      # of the request's logit scale; float32 rounding through a few layers
 BF16_TOL = 2e-2     # bfloat16 keeps 8 bits: eps 3.9e-3, a handful of roundings deep
 
-LENGTHS = {"A": [5, 17, 33, 70, 64, 100], "B": [1, 9, 40, 70, 129, 48], "C": [3, 65, 31, 96]}
+LENGTHS = {"A": [5, 17, 33, 70, 64, 100], "B": [1, 9, 40, 70, 129, 48], "C": [3, 65, 31, 96], "D": [2, 47, 80, 33, 16]}
 FAMILIES = ["whole", "decode_tail", "portions", "mixed"]
 
 
@@ -52,7 +52,7 @@ def run_replay(runner, steps, out_dir):
 
 
 @pytest.mark.parametrize("family", FAMILIES)
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_replay_host_path(tiny_models, tmp_path, name, family):
     m = tiny_models[name]
     prompts = trace_util.random_prompts(m["cfg"]["vocab_size"], LENGTHS[name], seed=11)
@@ -84,7 +84,7 @@ def test_mixed_trace_reuses_pages(tiny_models):
 @pytest.mark.gpu
 @pytest.mark.parametrize("family", FAMILIES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_replay_gpu(tiny_models, tmp_path, name, dtype, family):
     m = tiny_models[name]
     prompts = trace_util.random_prompts(m["cfg"]["vocab_size"], LENGTHS[name], seed=11)
