@@ -125,7 +125,7 @@ class HipBackend(KernelBackend):
         return y
 
     # ---- few-row products of the bfloat16 path: one fused kernel each
-    SKINNY_MAX_ROWS = 32      # above this the library product is faster than the fused kernel (measured at 24, 32, 48 rows)
+    SKINNY_MAX_ROWS = 32      # above this the split product or the library is faster than the fused kernel (measured at 24, 32, 48 rows)
     EPI_BF16, EPI_F32, EPI_ADD, EPI_SWIGLU = 0, 1, 2, 3
 
     def _skinny_ok(self, x, w, bias, rows=None) -> bool:
