@@ -15,8 +15,12 @@
 // or poisoned slots never reach the sums.
 #include "attention_bf16_common.hpp"
 
-constexpr int NW = D > 128 ? 2 : 4;    // waves per workgroup (bounded by the LDS the merge needs)
+constexpr int NW_SPLIT = D > 128 ? 2 : 4;    // waves per workgroup (bounded by the LDS the merge of the waves needs)
+// When rows and heads alone fill the GPU the context is not split and there is no second kernel; a workgroup then
+// has a whole context to read, and eight waves keep twice the loads in flight for it.
+constexpr int NW_WHOLE = D > 128 ? 2 : (D > 64 ? 4 : 8);
 
+template <int NW>
 __global__ void __launch_bounds__(NW * 64)
 decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* __restrict__ k_cache,
                         const bf16* __restrict__ v_cache, bf16* __restrict__ out, float* __restrict__ o_part,
@@ -289,7 +293,7 @@ merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ 
 
 MIE_EXPORT const char* attention_bf16_last_error() { return g_mie_error; }
 MIE_EXPORT int mie_attention_bf16_head_dim() { return D; }
-MIE_EXPORT int mie_decode_block_keys() { return BLOCK_KEYS * NW; }
+MIE_EXPORT int mie_decode_block_keys() { return BLOCK_KEYS * NW_SPLIT; }
 
 // q: token b is row b (single-token rows lead the flattened batch).  partition: keys per split, a
 // multiple of mie_decode_block_keys().  o_part [rows, Hq, splits, D] and lse_part [rows, Hq, splits]
@@ -302,17 +306,22 @@ MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_
   if (head_dim != D) MIE_FAIL("decode_attention: built for head_dim %d, called with %d", D, head_dim);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("decode_attention: %d query heads on %d kv heads", Hq, Hkv);
   if (page < 16 || page % 16) MIE_FAIL("decode_attention: page size %d (multiples of 16)", page);
-  if (partition <= 0 || partition % (BLOCK_KEYS * NW)) MIE_FAIL("decode_attention: partition %d is no multiple of %d", partition, BLOCK_KEYS * NW);
+  if (partition <= 0 || partition % (BLOCK_KEYS * NW_SPLIT)) MIE_FAIL("decode_attention: partition %d is no multiple of %d", partition, BLOCK_KEYS * NW_SPLIT);
   if (num_splits < 1 || num_splits > 65535) MIE_FAIL("decode_attention: %d splits", num_splits);
   if (num_splits > 1 && (!o_part || !lse_part)) MIE_FAIL("decode_attention: splits need partial buffers");
   if (q_stride < (long)Hq * D || (q_stride % 8) || ((uintptr_t)q % 16)) MIE_FAIL("decode_attention: q stride %ld / alignment", q_stride);
   if (max_blocks <= 0) MIE_FAIL("decode_attention: max_blocks %d", max_blocks);
   const int G = Hq / Hkv, head_tiles = (G + 15) / 16;
   if ((long)Hkv * head_tiles > 65535) MIE_FAIL("decode_attention: too many head tiles for the grid");
-  dim3 grid(rows, Hkv * head_tiles, num_splits), block(NW * 64);
-  hipLaunchKernelGGL(decode_attention_kernel, grid, block, 0, stream, (const bf16*)q, q_stride, (const bf16*)k_cache,
-                     (const bf16*)v_cache, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv,
-                     head_tiles, page, scale * 1.4426950408889634f, window, partition, num_splits);
+  dim3 grid(rows, Hkv * head_tiles, num_splits);
+  if (num_splits == 1 && NW_WHOLE != NW_SPLIT)
+    hipLaunchKernelGGL(decode_attention_kernel<NW_WHOLE>, grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)q, q_stride,
+                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, o_part, lse_part, block_tables, max_blocks,
+                       positions, Hq, Hkv, head_tiles, page, scale * 1.4426950408889634f, window, partition, num_splits);
+  else
+    hipLaunchKernelGGL(decode_attention_kernel<NW_SPLIT>, grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)q, q_stride,
+                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, o_part, lse_part, block_tables, max_blocks,
+                       positions, Hq, Hkv, head_tiles, page, scale * 1.4426950408889634f, window, partition, num_splits);
   MIE_CHECK_LAUNCH("decode_attention");
   if (num_splits > 1) {
     hipLaunchKernelGGL(merge_splits_kernel, dim3(rows * Hq), dim3(64), 0, stream, o_part, lse_part, (bf16*)out, num_splits);

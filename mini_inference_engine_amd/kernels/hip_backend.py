@@ -415,6 +415,7 @@ class HipBackend(KernelBackend):
 
     # workgroups the decode attention kernel should at least be spread over (two per compute unit)
     DECODE_TARGET_WORKGROUPS = 512
+    DECODE_WHOLE_WORKGROUPS = 256
 
     def decode_splits(self, rows: int, Hq: int, Hkv: int, context_bound: int, window, block_keys: int):
         """(keys per split, number of splits) for single-token rows: split the context only as far
@@ -424,7 +425,9 @@ class HipBackend(KernelBackend):
             context_bound = min(context_bound, window + 32)
         base = rows * Hkv * -(-(Hq // Hkv) // 16)
         most = max(1, -(-context_bound // block_keys))
-        splits = max(1, min(-(-self.DECODE_TARGET_WORKGROUPS // base), most))
+        # rows and heads that give every compute unit a workgroup are not split: no partial results, no merge
+        target = self.DECODE_TARGET_WORKGROUPS if base < self.DECODE_WHOLE_WORKGROUPS else base
+        splits = max(1, min(-(-target // base), most))
         partition = -(-(-(-context_bound // splits)) // block_keys) * block_keys
         return partition, max(1, -(-context_bound // partition))
 
