@@ -28,10 +28,13 @@
 // scale * log2(e); l is a per-lane partial sum, joined over a query's two lanes at the end.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-// Waves a workgroup: 8 where that still gives a workgroup to every compute unit (twice the queries share
-// each block that is brought in: at head size 128 and 8,192 tokens 0.82 against 0.40 PFLOP/s), else 4
-// (and always 4 at head sizes above 128, where eight waves do not fit the registers).
+// Waves a workgroup, at head sizes up to 128 (above, eight waves do not fit the registers: always 4):
+// 8 over twice the queries where that still gives a workgroup to every compute unit (twice the queries share
+// each block that is brought in: at head size 128 and 8,192 tokens 0.82 against 0.40 PFLOP/s); for shorter
+// rows 8 in two halves over the keys, on the grid of 4: a wave's chain of blocks is half as long and every
+// SIMD has two waves (2,048 tokens at head size 64: 47 against 56 us).
 constexpr int PF_MAX_WAVES = D > 128 ? 4 : 8;
+constexpr bool PF_KEY_HALVES = D <= 128;            // (at 128 the two halves' kernel does not fit the registers)
 constexpr int PF_QW = 32;                           // queries a wave owns
 constexpr int PF_BK = 64;                           // keys a step
 constexpr int KS16 = D / 16;                        // 16-dim steps of q . k
@@ -62,7 +65,10 @@ __device__ __forceinline__ float pair_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-template <int PF_WAVES>
+// KS = 2: the waves form two halves that take the even and the odd 64-key blocks of the same queries (a step
+// brings 128 keys in, each half computes its 64) and join their results at the end: half the blocks a wave
+// for rows too short to give every SIMD two waves otherwise.
+template <int PF_WAVES, int KS>
 __global__ void __launch_bounds__(PF_WAVES * 64)
 prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* __restrict__ k_cache,
                          const bf16* __restrict__ v_cache, bf16* __restrict__ out,
@@ -71,7 +77,11 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
                          int page, float scale_log2, int window) {
   extern __shared__ __align__(16) unsigned char pf_lds[];
   constexpr int PF_THREADS = PF_WAVES * 64;
-  constexpr int PF_PPT = (PF_PIECES + PF_THREADS - 1) / PF_THREADS;       // pieces a thread carries
+  constexpr int SUB_WAVES = PF_WAVES / KS;                   // waves of one half
+  constexpr int FK = PF_BK * KS;                             // keys a step brings in
+  constexpr int T16 = FK / 16;                               // 16-key pieces of a value row a step
+  constexpr int KPIECES = KS * PF_KPIECES, PIECES = KS * PF_PIECES;
+  constexpr int PF_PPT = (PIECES + PF_THREADS - 1) / PF_THREADS;          // pieces a thread carries
   // Which (stretch pair, row, kv head) this workgroup takes.  Workgroups go to the eight XCDs in turn, in
   // launch order with x fastest, and every XCD has an L2 of its own: all workgroups of one kv head read
   // the same keys and values, so they are placed on one XCD (or on 8 / Z of them when there are fewer
@@ -96,7 +106,7 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
   }
   const int row = first_row + by;
   const int G = Hq / Hkv;
-  const int waves_q = PF_WAVES / waves_h;                     // query tiles a workgroup serves at a time
+  const int waves_q = SUB_WAVES / waves_h;                    // query tiles a workgroup serves at a time
   const int head_chunks = (G + waves_h - 1) / waves_h;
   const int kvh = bz / head_chunks, hc = bz - kvh * head_chunks;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -106,12 +116,13 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
   const int STRETCH = PF_QW * waves_q;
   const int NS = (q_len + STRETCH - 1) / STRETCH;              // stretches of this row
   if (bx >= (NS + 1) / 2) return;               // the whole workgroup, before any barrier
-  const int wh = wave % waves_h, wq = wave / waves_h;
+  const int wk = wave / SUB_WAVES, wsub = wave - wk * SUB_WAVES;  // which half, and the wave's place in it
+  const int wh = wsub % waves_h, wq = wsub / waves_h;
   const int* bt = block_tables + (size_t)row * max_blocks;
 
   // rows of dims beyond D in the value buffers are never written: zero them once
   if (D % 32 != 0) {
-    for (int i = tid; i < 2 * 16 * (PF_VROW / 16); i += PF_THREADS) {
+    for (int i = tid; i < 2 * KS * 16 * (PF_VROW / 16); i += PF_THREADS) {
       const int buf = i / (16 * (PF_VROW / 16)), rest = i % (16 * (PF_VROW / 16));
       *reinterpret_cast<uint4*>(pf_lds + buf * PF_BUF + PF_KBYTES + (D + rest / (PF_VROW / 16)) * PF_VROW +
                                 (rest % (PF_VROW / 16)) * 16) = make_uint4(0, 0, 0, 0);
@@ -173,7 +184,9 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
       blk = blk < last_blk ? blk : last_blk;           // beyond the last block: the last one again
       {
         const int d = blk - walk_start;
-        const int adv = (d >= page ? 1 : 0) + (d >= 2 * page ? 1 : 0) + (d >= 3 * page ? 1 : 0) + (d >= 4 * page ? 1 : 0);
+        int adv = 0;
+#pragma unroll
+        for (int k = 1; k <= T16; ++k) adv += d >= k * page ? 1 : 0;
         walk_start += adv * page;
         walk_idx += adv;
       }
@@ -181,16 +194,17 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
       for (int i = 0; i < PF_PPT; ++i) {
         const int c = tid + PF_THREADS * i;
         int key;
-        if (c < PF_KPIECES) {                          // keys: dims 16 j .. 16 j + 15 of key c / (D / 16)
+        if (c < KPIECES) {                             // keys: dims 16 j .. 16 j + 15 of key c / (D / 16)
           key = blk + c / (D / 16);
           key = key < kmax ? key : kmax;
-        } else {                                       // values: keys 16 t .. 16 t + 15 of one dim, t = c % 4
-          key = blk + ((c - PF_KPIECES) & 3) * 16;
+        } else {                                       // values: keys 16 t .. 16 t + 15 of one dim, t = c % T16
+          key = blk + ((c - KPIECES) % T16) * 16;
           key = key < (kmax & ~15) ? key : (kmax & ~15);
         }
         const int rel = key - walk_start;
-        const int w = (rel >= page ? 1 : 0) + (rel >= 2 * page ? 1 : 0) + (rel >= 3 * page ? 1 : 0) +
-                      (rel >= 4 * page ? 1 : 0);
+        int w = 0;
+#pragma unroll
+        for (int k = 1; k <= T16; ++k) w += rel >= k * page ? 1 : 0;
         Wh.pg[i] = bt[walk_idx + w];
         Wh.off[i] = rel - w * page;
       }
@@ -200,27 +214,29 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
       for (int i = 0; i < PF_PPT; ++i) {
         const int c = tid + PF_THREADS * i;
         const bf16* src = nullptr;
-        if (c < PF_KPIECES)
+        if (c < KPIECES)
           src = k_cache + (((size_t)Wh.pg[i] * Hkv + kvh) * page + Wh.off[i]) * D + (c % (D / 16)) * 16;
-        else if (c < PF_PIECES)
-          src = v_cache + (((size_t)Wh.pg[i] * Hkv + kvh) * D + ((c - PF_KPIECES) >> 2)) * page + Wh.off[i];
+        else if (c < PIECES)
+          src = v_cache + (((size_t)Wh.pg[i] * Hkv + kvh) * D + (c - KPIECES) / T16) * page + Wh.off[i];
         if (src) {
           P.lo[i] = *reinterpret_cast<const uint4*>(src);
           P.hi[i] = *reinterpret_cast<const uint4*>(src + 8);
         }
       }
     };
-    auto stash = [&](Pieces& P, int buf, int blk) {
-      unsigned char* base = pf_lds + buf * PF_BUF;
+    // a set of buffers holds one step: KS blocks of 64 keys, one buffer each
+    auto stash = [&](Pieces& P, int set, int blk) {
+      unsigned char* base = pf_lds + set * KS * PF_BUF;
 #pragma unroll
       for (int i = 0; i < PF_PPT; ++i) {
         const int c = tid + PF_THREADS * i;
-        if (c < PF_KPIECES) {
-          unsigned char* at = base + (c / (D / 16)) * PF_KROW + (c % (D / 16)) * 32;
+        if (c < KPIECES) {
+          const int key = c / (D / 16);
+          unsigned char* at = base + (key / PF_BK) * PF_BUF + (key % PF_BK) * PF_KROW + (c % (D / 16)) * 32;
           *reinterpret_cast<uint4*>(at) = P.lo[i];
           *reinterpret_cast<uint4*>(at + 16) = P.hi[i];
-        } else if (c < PF_PIECES) {
-          const int cv = c - PF_KPIECES, t = cv & 3;
+        } else if (c < PIECES) {
+          const int cv = c - KPIECES, t = cv % T16, dim = cv / T16;
           uint32_t w[8] = {P.lo[i].x, P.lo[i].y, P.lo[i].z, P.lo[i].w, P.hi[i].x, P.hi[i].y, P.hi[i].z, P.hi[i].w};
           const int key0 = blk + t * 16;
           if (key0 + 15 > kmax) {
@@ -233,17 +249,17 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
           }
           // within a row the keys stand in the order the second product wants them: for lane half 0 keys
           // 16 t + {0..3, 8..11}, for lane half 1 keys 16 t + {4..7, 12..15}, each one 16-byte read
-          unsigned char* at = base + PF_KBYTES + (cv >> 2) * PF_VROW + t * 32;
+          unsigned char* at = base + (t / 4) * PF_BUF + PF_KBYTES + dim * PF_VROW + (t % 4) * 32;
           *reinterpret_cast<uint4*>(at) = make_uint4(w[0], w[1], w[4], w[5]);
           *reinterpret_cast<uint4*>(at + 16) = make_uint4(w[2], w[3], w[6], w[7]);
         }
       }
     };
 
-    // ---- one block of 64 keys for the wave's tile
-    auto compute = [&](int buf, int blk) {
-      const unsigned char* Kb = pf_lds + buf * PF_BUF + col * PF_KROW + g * 16;
-      const unsigned char* Vb = pf_lds + buf * PF_BUF + PF_KBYTES + col * PF_VROW + g * 16;
+    // ---- one block of 64 keys for the wave's tile: the wave's half of the step in set `set`
+    auto compute = [&](int set, int blk) {
+      const unsigned char* Kb = pf_lds + (set * KS + wk) * PF_BUF + col * PF_KROW + g * 16;
+      const unsigned char* Vb = pf_lds + (set * KS + wk) * PF_BUF + PF_KBYTES + col * PF_VROW + g * 16;
       f32x16 S[2];
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
@@ -325,42 +341,72 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
         }
     };
 
-    // ---- the blocks, two LDS buffers and two sets of registers: while block i is computed, block i + 1
-    // sits in registers (asked for an iteration ago, stored to the LDS after the computing), block i + 2 is
-    // on its way from memory and the pages of block i + 3 are looked up.  One barrier a block.
+    // ---- the steps, two sets of LDS buffers and two sets of registers: while step i is computed, step i + 1
+    // sits in registers (asked for an iteration ago, stored to the LDS after the computing), step i + 2 is
+    // on its way from memory and the pages of step i + 3 are looked up.  One barrier a step.
     Where wh_;
     Pieces pa, pb_;
     lookup(wh_, blk0);
-    fetch(pa, wh_);                                    // block 0
-    lookup(wh_, blk0 + PF_BK);
-    fetch(pb_, wh_);                                   // block 1 (clamped into the row if there is none)
-    lookup(wh_, blk0 + 2 * PF_BK);
+    fetch(pa, wh_);                                    // step 0
+    lookup(wh_, blk0 + FK);
+    fetch(pb_, wh_);                                   // step 1 (clamped into the row if there is none)
+    lookup(wh_, blk0 + 2 * FK);
     __syncthreads();                                   // the previous stretch is done with the buffers
     stash(pa, 0, blk0);
     __syncthreads();
+    const int mine_off = wk * PF_BK;                   // this wave's block within a step
     auto mine = [&](int blk) { return blk <= wave_kmax && blk + PF_BK > wave_kmin; };
-    for (int blk = blk0; blk <= kmax; blk += 2 * PF_BK) {      // every condition is uniform over the workgroup
-      // block blk from buffer 0; pb_ holds block blk + 64; pa is free for block blk + 128
-      if (blk + 2 * PF_BK <= kmax) {
+    for (int blk = blk0; blk <= kmax; blk += 2 * FK) {         // every condition is uniform over the workgroup
+      // step blk from set 0; pb_ holds step blk + FK; pa is free for step blk + 2 FK
+      if (blk + 2 * FK <= kmax) {
         fetch(pa, wh_);
-        lookup(wh_, blk + 3 * PF_BK);
+        lookup(wh_, blk + 3 * FK);
       }
-      if (mine(blk)) compute(0, blk);
-      if (blk + PF_BK > kmax) break;                   // (no barrier needed: nothing reads the LDS after this)
-      stash(pb_, 1, blk + PF_BK);
+      if (mine(blk + mine_off)) compute(0, blk + mine_off);
+      if (blk + FK > kmax) break;
+      stash(pb_, 1, blk + FK);
       __syncthreads();
-      // block blk + 64 from buffer 1; pa holds block blk + 128; pb_ is free for block blk + 192
-      if (blk + 3 * PF_BK <= kmax) {
+      // step blk + FK from set 1; pa holds step blk + 2 FK; pb_ is free for step blk + 3 FK
+      if (blk + 3 * FK <= kmax) {
         fetch(pb_, wh_);
-        lookup(wh_, blk + 4 * PF_BK);
+        lookup(wh_, blk + 4 * FK);
       }
-      if (mine(blk + PF_BK)) compute(1, blk + PF_BK);
-      if (blk + 2 * PF_BK <= kmax) stash(pa, 0, blk + 2 * PF_BK);
+      if (mine(blk + FK + mine_off)) compute(1, blk + FK + mine_off);
+      if (blk + 2 * FK <= kmax) stash(pa, 0, blk + 2 * FK);
       __syncthreads();
     }
 
+    if (KS == 2) {
+      // The halves join: the second half's state goes through the LDS (item i of lane l at 4 (64 i + l), a
+      // region a wave), the first half rescales both to the common maximum.  l and O are per-lane partial
+      // sums, m is the same in a query's two lanes.
+      float* xch = reinterpret_cast<float*>(pf_lds) + wsub * (64 * (2 + 16 * DT32)) + lane;
+      __syncthreads();                                 // everybody is done with the keys and values
+      if (wk == 1) {
+        xch[0] = m;
+        xch[64] = l;
+#pragma unroll
+        for (int dt = 0; dt < DT32; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) xch[64 * (2 + dt * 16 + i)] = O[dt][i];
+      }
+      __syncthreads();
+      if (wk == 0) {
+        const float m1 = xch[0], l1 = xch[64];
+        const float mj = max_nn(m, m1);
+        // a half may have seen no key of a query (m = -inf, sums 0): it counts for nothing
+        const float a0 = m == -INFINITY ? 0.f : fast_exp2(m - mj);
+        const float a1 = m1 == -INFINITY ? 0.f : fast_exp2(m1 - mj);
+        l = l * a0 + l1 * a1;
+#pragma unroll
+        for (int dt = 0; dt < DT32; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) O[dt][i] = O[dt][i] * a0 + xch[64 * (2 + dt * 16 + i)] * a1;
+      }
+    }
+
     const float total = pair_sum(l);
-    if (q_ok) {
+    if (q_ok && wk == 0) {
       const float inv = 1.0f / total;
       bf16* op = out + ((size_t)qtok * Hq + head) * D + 4 * g;
 #pragma unroll
@@ -395,19 +441,8 @@ MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k
     MIE_FAIL("prefill_attention: q stride %ld / alignment", q_stride);
   if (max_blocks <= 0) MIE_FAIL("prefill_attention: max_blocks %d", max_blocks);
   const int G = Hq / Hkv;
-  constexpr int lds_bytes = 2 * PF_BUF;
-  static bool lds_allowed[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) MIE_FAIL("prefill_attention: no current device");
-  if (lds_bytes > 64 * 1024 && !lds_allowed[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_attention_kernel<4>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e == hipSuccess && PF_MAX_WAVES == 8)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_attention_kernel<PF_MAX_WAVES>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) MIE_FAIL("prefill_attention: %d bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
-    lds_allowed[dev] = true;
-  }
   // the grid for `waves` waves a workgroup: waves side by side over the heads of a group (a power of two), the rest
   // over 32-query tiles; a workgroup takes a late stretch and an early one
   auto plan = [&](int waves, int* waves_h, dim3* grid) {
@@ -420,20 +455,40 @@ MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k
     *grid = dim3((unsigned)((stretches + 1) / 2), rows, Hkv * head_chunks);
     return (long)grid->x * grid->y * grid->z;
   };
-  int waves = 4, waves_h;
+  // Eight waves over twice the queries where that still gives every compute unit a workgroup; else, at head
+  // sizes that leave room, eight waves in two halves over the keys (the grid of four waves); else four waves.
+  enum { FOUR, EIGHT_QUERIES, EIGHT_KEYS } kind = FOUR;
+  int waves_h;
   dim3 grid;
-  if (PF_MAX_WAVES == 8 && plan(8, &waves_h, &grid) >= (D >= 128 ? 128 : 256)) waves = 8;
-  plan(waves, &waves_h, &grid);
+  if (PF_MAX_WAVES == 8) {
+    // (at head size 128 a compute unit holds one workgroup of the two-halves kind: more of them than compute
+    // units would run in two rounds, the second half empty)
+    const long n8 = plan(8, &waves_h, &grid), n4 = plan(4, &waves_h, &grid);
+    kind = n8 >= 256 || (D >= 128 && n4 > 256) ? EIGHT_QUERIES : EIGHT_KEYS;
+  }
+  plan(kind == EIGHT_QUERIES ? 8 : 4, &waves_h, &grid);
   if (grid.y > 65535 || grid.z > 65535) MIE_FAIL("prefill_attention: grid too large (%d rows)", rows);
   const float scale_log2 = scale * 1.4426950408889634f;
-  if (waves == 8)
-    hipLaunchKernelGGL(prefill_attention_kernel<PF_MAX_WAVES>, grid, dim3(PF_MAX_WAVES * 64), lds_bytes, stream, (const bf16*)q,
-                       q_stride, (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, block_tables, max_blocks, row_start,
-                       row_position, first_row, Hq, Hkv, waves_h, page, scale_log2, window);
-  else
-    hipLaunchKernelGGL(prefill_attention_kernel<4>, grid, dim3(256), lds_bytes, stream, (const bf16*)q, q_stride,
-                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, block_tables, max_blocks, row_start,
-                       row_position, first_row, Hq, Hkv, waves_h, page, scale_log2, window);
+  // more LDS than a kernel gets by default is asked for once per kernel and device
+  static bool lds_allowed[3][64] = {};
+  auto launch = [&](auto kernel, int waves, int lds_bytes) -> int {
+    if (lds_bytes > 64 * 1024 && !lds_allowed[kind][dev]) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      if (e != hipSuccess) MIE_FAIL("prefill_attention: %d bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
+      lds_allowed[kind][dev] = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(waves * 64), lds_bytes, stream, (const bf16*)q, q_stride, (const bf16*)k_cache,
+                       (const bf16*)v_cache, (bf16*)out, block_tables, max_blocks, row_start, row_position, first_row, Hq, Hkv,
+                       waves_h, page, scale_log2, window);
+    return 0;
+  };
+  int rc = 0;
+  if constexpr (PF_MAX_WAVES == 8) {
+    if (kind == EIGHT_QUERIES) rc = launch(prefill_attention_kernel<8, 1>, 8, 2 * PF_BUF);
+    if (kind == EIGHT_KEYS) rc = launch(prefill_attention_kernel<8, 2>, 8, 4 * PF_BUF);
+  }
+  if (kind == FOUR) rc = launch(prefill_attention_kernel<4, 1>, 4, 2 * PF_BUF);
+  if (rc) return rc;
   MIE_CHECK_LAUNCH("prefill_attention");
   return 0;
 }

@@ -122,6 +122,95 @@ rotary_kv_store_bf16x8_kernel(bf16* __restrict__ qkv, long row_stride, const int
   }
 }
 
+// The same from the projection's float32 sums, for steps of many tokens (bfloat16 caches): q and k are
+// rounded once, after the rotation.  sums [tokens, ld] float32 (q heads, k heads, v heads); q_out [tokens, ldq]
+// bfloat16 gets the rotated q; rotated k and v go to their slots.  Rotation over the whole head.
+// grid (ceil(tokens / 16), ceil(heads / 4)): a workgroup takes 16 tokens of 4 heads.  Rotary heads: a thread
+// takes four pairs (16 bytes of sums on each side).  Value heads are turned in the LDS ([dim][token]), so that
+// a thread owns one dim's 16 tokens: where the 16 tokens are one run of 16
+// slots of one page starting at a multiple of 16 (a prompt written from a page's start), they go out as 32
+// contiguous bytes; otherwise one by one.
+constexpr int RS_TOK = 16, RS_HEADS = 4, RS_VROW = RS_TOK + 8;      // LDS row of a dim: 16 tokens + padding (bf16)
+
+__device__ __forceinline__ uint32_t rs_pack(float a, float b) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, __float2bfloat16(a)) | ((uint32_t)__builtin_bit_cast(uint16_t, __float2bfloat16(b)) << 16);
+}
+
+__global__ void __launch_bounds__(256)
+rotary_kv_store_sums_kernel(const float* __restrict__ sums, long ld, bf16* __restrict__ q_out, long ldq,
+                            const int* __restrict__ positions, const float* __restrict__ cos_t,
+                            const float* __restrict__ sin_t, const int* __restrict__ slots, bf16* __restrict__ k_cache,
+                            bf16* __restrict__ v_cache, int Hq, int Hkv, int D, int page, int tokens) {
+  extern __shared__ __align__(16) unsigned char rs_lds[];
+  __shared__ int s_slot[RS_TOK], s_pos[RS_TOK];
+  bf16* vt = reinterpret_cast<bf16*>(rs_lds);                       // [RS_HEADS * D][RS_VROW]
+  const int t0 = blockIdx.x * RS_TOK, n = tokens - t0 < RS_TOK ? tokens - t0 : RS_TOK;
+  const int h0 = blockIdx.y * RS_HEADS, heads = Hq + 2 * Hkv;
+  const int nh = heads - h0 < RS_HEADS ? heads - h0 : RS_HEADS;
+  if (threadIdx.x < RS_TOK) {
+    const int t = t0 + (threadIdx.x < n ? threadIdx.x : 0);
+    s_slot[threadIdx.x] = slots[t];
+    s_pos[threadIdx.x] = positions[t];
+  }
+  __syncthreads();
+  const int half = D >> 1, groups = half >> 2;                      // four pairs a thread
+  // ---- q and k heads of this chunk
+  const int rot_heads = h0 >= Hq + Hkv ? 0 : (Hq + Hkv - h0 < nh ? Hq + Hkv - h0 : nh);
+  for (int w = threadIdx.x; w < n * rot_heads * groups; w += blockDim.x) {
+    const int jg = w % groups, rest = w / groups, hh = rest % rot_heads, i = rest / rot_heads;
+    const int head = h0 + hh, j = jg << 2, t = t0 + i;
+    const float* src = sums + (size_t)t * ld + (size_t)head * D;
+    const float4 a = *reinterpret_cast<const float4*>(src + j), b = *reinterpret_cast<const float4*>(src + j + half);
+    const float4 c = *reinterpret_cast<const float4*>(cos_t + (size_t)s_pos[i] * half + j);
+    const float4 sn = *reinterpret_cast<const float4*>(sin_t + (size_t)s_pos[i] * half + j);
+    uint2 o1, o2;
+    o1.x = rs_pack(a.x * c.x - b.x * sn.x, a.y * c.y - b.y * sn.y);
+    o1.y = rs_pack(a.z * c.z - b.z * sn.z, a.w * c.w - b.w * sn.w);
+    o2.x = rs_pack(b.x * c.x + a.x * sn.x, b.y * c.y + a.y * sn.y);
+    o2.y = rs_pack(b.z * c.z + a.z * sn.z, b.w * c.w + a.w * sn.w);
+    bf16* dst;
+    if (head < Hq) {
+      dst = q_out + (size_t)t * ldq + (size_t)head * D;
+    } else {
+      const int slot = s_slot[i];
+      dst = k_cache + (((size_t)(slot / page) * Hkv + (head - Hq)) * page + (size_t)(slot % page)) * D;
+    }
+    *reinterpret_cast<uint2*>(dst + j) = o1;
+    *reinterpret_cast<uint2*>(dst + j + half) = o2;
+  }
+  // ---- v heads of this chunk (the condition is the same for the whole workgroup)
+  const int v_first = h0 > Hq + Hkv ? h0 : Hq + Hkv;                // first value head of this chunk
+  const int v_heads = h0 + nh - v_first;
+  if (v_heads <= 0) return;
+  const int d4 = D >> 2;
+  for (int w = threadIdx.x; w < n * v_heads * d4; w += blockDim.x) {
+    const int dg = w % d4, rest = w / d4, hh = rest % v_heads, i = rest / v_heads;
+    const float4 a = *reinterpret_cast<const float4*>(sums + (size_t)(t0 + i) * ld + (size_t)(v_first + hh) * D + dg * 4);
+    bf16* at = vt + (size_t)(hh * D + dg * 4) * RS_VROW + i;
+    at[0] = __float2bfloat16(a.x);
+    at[RS_VROW] = __float2bfloat16(a.y);
+    at[2 * RS_VROW] = __float2bfloat16(a.z);
+    at[3 * RS_VROW] = __float2bfloat16(a.w);
+  }
+  __syncthreads();
+  bool run = n == RS_TOK && (s_slot[0] & 15) == 0 && s_slot[0] % page + RS_TOK <= page;
+  for (int i = 1; i < RS_TOK; ++i) run = run && s_slot[i] == s_slot[0] + i;
+  for (int w = threadIdx.x; w < v_heads * D; w += blockDim.x) {
+    const int hh = w / D, d = w - hh * D, kvh = v_first + hh - Hq - Hkv;
+    const bf16* from = vt + (size_t)w * RS_VROW;
+    if (run) {
+      bf16* dst = v_cache + (((size_t)(s_slot[0] / page) * Hkv + kvh) * D + d) * page + (size_t)(s_slot[0] % page);
+      *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(from);
+      *reinterpret_cast<uint4*>(dst + 8) = *reinterpret_cast<const uint4*>(from + 8);
+    } else {
+      for (int i = 0; i < n; ++i) {
+        const int slot = s_slot[i];
+        v_cache[(((size_t)(slot / page) * Hkv + kvh) * D + d) * page + (size_t)(slot % page)] = from[i];
+      }
+    }
+  }
+}
+
 MIE_EXPORT const char* rope_kv_last_error() { return g_mie_error; }
 
 MIE_EXPORT int mie_rotary_kv_store(void* qkv, int dtype, long row_stride, const int* positions, const float* cos_t,
@@ -146,5 +235,26 @@ MIE_EXPORT int mie_rotary_kv_store(void* qkv, int dtype, long row_stride, const 
   else
     MIE_FAIL("rotary_kv_store: dtype code %d", dtype);
   MIE_CHECK_LAUNCH("rotary_kv_store");
+  return 0;
+}
+
+// sums [tokens, ld] float32, the q/k/v projection before rounding; bfloat16 q_out and caches; head_dim a
+// multiple of 8, rotation over the whole head.
+MIE_EXPORT int mie_rotary_kv_store_sums(const float* sums, long ld, void* q_out, long ldq, const int* positions,
+                                        const float* cos_t, const float* sin_t, const int* slots, void* k_cache,
+                                        void* v_cache, int Hq, int Hkv, int D, int page, int tokens, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (D <= 0 || (D & 7)) MIE_FAIL("rotary_kv_store_sums: head_dim %d must be a multiple of 8", D);
+  if (Hq <= 0 || Hkv <= 0 || page < 16 || (page & 15)) MIE_FAIL("rotary_kv_store_sums: heads %d / %d, page %d", Hq, Hkv, page);
+  if (!sums || !q_out || !positions || !cos_t || !sin_t || !slots || !k_cache || !v_cache) MIE_FAIL("rotary_kv_store_sums: null operand");
+  if (ld < (long)(Hq + 2 * Hkv) * D || (ld & 3) || ldq < (long)Hq * D || (ldq & 3)) MIE_FAIL("rotary_kv_store_sums: leading dims %ld, %ld", ld, ldq);
+  if ((((uintptr_t)sums | (uintptr_t)cos_t | (uintptr_t)sin_t | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) || ((uintptr_t)q_out & 7))
+    MIE_FAIL("rotary_kv_store_sums: operands must be 16-byte aligned");
+  const int lds_bytes = RS_HEADS * D * RS_VROW * (int)sizeof(bf16);
+  if (lds_bytes > 64 * 1024) MIE_FAIL("rotary_kv_store_sums: head_dim %d needs %d bytes of LDS", D, lds_bytes);
+  dim3 grid((tokens + RS_TOK - 1) / RS_TOK, (Hq + 2 * Hkv + RS_HEADS - 1) / RS_HEADS);
+  hipLaunchKernelGGL(rotary_kv_store_sums_kernel, grid, dim3(256), lds_bytes, stream, sums, ld, (bf16*)q_out, ldq, positions, cos_t,
+                     sin_t, slots, (bf16*)k_cache, (bf16*)v_cache, Hq, Hkv, D, page, tokens);
+  MIE_CHECK_LAUNCH("rotary_kv_store_sums");
   return 0;
 }

@@ -312,6 +312,22 @@ class HipBackend(KernelBackend):
         fused = can_rope and self._skinny_ok(x, w_qkv, None)
         if not fused and can_rope and self._mid_ok(x, w_qkv, None) and self.act_dtype == torch.bfloat16:
             return self._mid_rotary_kv_store(x, w_qkv, positions, cos, sin, Hq, Hkv, D, k_cache, v_cache, slot_mapping)
+        if (not fused and can_rope and not self.true_fp32 and self.act_dtype == torch.bfloat16
+                and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16):
+            # many rows: library product with float32 sums, then rotary and cache write from those sums (q and k
+            # are rounded to bfloat16 once, after the rotation)
+            self._on_device(x, w_qkv)
+            self._on_device(positions, cos, sin, k_cache, v_cache, slot_mapping)
+            M, K = x.shape
+            page = self._check_rope_operands("linear_rotary_kv_store", M, K, w_qkv, positions, cos, sin, Hq, Hkv, D,
+                                             k_cache, v_cache, slot_mapping)
+            sums = torch.mm(x, w_qkv.t(), out_dtype=torch.float32)
+            q = torch.empty((M, Hq * D), dtype=torch.bfloat16, device=x.device)
+            lib = self.lib("rope_kv")
+            library.check(lib, lib.mie_rotary_kv_store_sums(
+                _ptr(sums), sums.stride(0), _ptr(q), q.stride(0), _ptr(positions), _ptr(cos), _ptr(sin),
+                _ptr(slot_mapping), _ptr(k_cache), _ptr(v_cache), Hq, Hkv, D, page, M, self._stream()))
+            return q
         if not fused:
             return super().linear_rotary_kv_store(x, w_qkv, positions, cos, sin, rotary_dim, Hq, Hkv, D, k_cache,
                                                   v_cache, slot_mapping)

@@ -15,6 +15,7 @@ register_kernel_module("embed_norm", {
 })
 register_kernel_module("rope_kv", {
     "mie_rotary_kv_store": [P, I, L, P, P, P, I, I, I, I, P, P, P, I, I, P],
+    "mie_rotary_kv_store_sums": [P, L, P, L, P, P, P, P, P, P, I, I, I, I, I, P],
 })
 register_kernel_module("gemm", {
     "mie_gemm_nt": [P, I, L, P, I, L, P, I, L, P, I, I, I, P],

@@ -265,6 +265,49 @@ def test_mid_projection_rotary_store(engine_ops, geom, M):
     assert torch.equal(kc[0].float(), kc_ref[0]) and torch.equal(vc[0].float(), vc_ref[0]), "untouched pages stay untouched"
 
 
+@pytest.mark.parametrize("geom", [(2, 1, 16), (3, 1, 32), (4, 2, 48), (32, 4, 64), (5, 5, 96), (8, 2, 128), (2, 1, 256)])
+@pytest.mark.parametrize("slots_kind", ["page starts", "mid page", "scattered"])
+def test_many_row_projection_rotary_store(engine_ops, geom, slots_kind):
+    """More than 128 rows: library product with float32 sums, then one kernel for rotary + cache write that
+    reads those sums (16 tokens and 4 heads a workgroup; values turned in the LDS).  Slots in runs from a
+    page's start (the 32-byte path), runs from the middle of a page, and scattered; a token count that is no
+    multiple of 16; pages of 16 and of 32."""
+    from mini_inference_engine_amd.parts.rope import rotary_tables
+    Hq, Hkv, D = geom
+    o = engine_ops
+    M, K = 203, 264
+    page = 32 if D == 48 else 16
+    pages = 2 + -(-(M + page) // page)
+    torch.manual_seed(D + len(slots_kind))
+    cos, sin = (t.to(DEV) for t in rotary_tables(10000.0, D, 300))
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn((Hq + 2 * Hkv) * D, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    assert not o._mid_ok(x, w, None) and not o._skinny_ok(x, w, None)
+    pos = torch.randint(0, 300, (M,), device=DEV, dtype=torch.int32)
+    if slots_kind == "page starts":
+        slots = torch.arange(M, device=DEV, dtype=torch.int32) + page
+    elif slots_kind == "mid page":
+        slots = torch.arange(M, device=DEV, dtype=torch.int32) + page + 5
+    else:
+        slots = (torch.randperm((pages - 1) * page, device=DEV)[:M] + page).to(torch.int32)
+    kc, vc = make_cache(pages, Hkv, page, D, torch.bfloat16)
+    kc_ref, vc_ref = kc.float(), vc.float()
+    qkv_ref = ref.ref_linear(x, w, None, torch.float32)
+    ref.ref_rotary_kv_store(qkv_ref, pos, cos, sin, D, Hq, Hkv, D, kc_ref, vc_ref, slots)
+    out = o.linear_rotary_kv_store(x, w, pos, cos, sin, D, Hq, Hkv, D, kc, vc, slots)
+    assert tuple(out.shape) == (M, Hq * D), "q alone comes back"
+    # one rounding, of the rotated float32 value
+    torch.testing.assert_close(out.float(), qkv_ref[:, :Hq * D], atol=1e-2, rtol=8e-3)
+    torch.testing.assert_close(kc.float(), kc_ref, atol=1e-2, rtol=8e-3)
+    torch.testing.assert_close(vc.float(), vc_ref, atol=1e-2, rtol=8e-3)
+    assert torch.equal(kc[0].float(), kc_ref[0]) and torch.equal(vc[0].float(), vc_ref[0]), "untouched pages stay untouched"
+    written = torch.zeros(pages * page, dtype=torch.bool, device=DEV)
+    written[slots.long()] = True
+    keep = ~written.view(pages, page)
+    assert torch.equal(kc.float().permute(0, 2, 1, 3)[keep], kc_ref.permute(0, 2, 1, 3)[keep]), "other slots' keys stay"
+    assert torch.equal(vc.float().permute(0, 3, 1, 2)[keep], vc_ref.permute(0, 3, 1, 2)[keep]), "other slots' values stay"
+
+
 def test_lazy_norm_input_adds_once(ops):
     """A Normed handed to linear: what is pending is added to the stream exactly once, however often it is used."""
     o = ops[torch.bfloat16]
