@@ -263,7 +263,14 @@ class HipBackend(KernelBackend):
             # library matrix product, 32-bit accumulation, as the reference's F.linear.  What goes into the
             # float32 stream or out as logits leaves the product in float32: the sums are not rounded to
             # bfloat16 on their way there, whatever the number of rows.
-            if bias is None and (sink is not None or out_dtype == torch.float32):
+            if bias is None and sink is not None:
+                # the product adds its float32 sums to the stream itself (C = C + A B in place): the stream is
+                # not read and written once more by a kernel of its own
+                torch.ops.aten.addmm.dtype_out(sink.stream, x, w.t(), torch.float32, out=sink.stream)
+                if sink.norm_weight is None:
+                    return None
+                return Normed(self, None, sink.stream, sink.norm_weight, sink.norm_eps)
+            if bias is None and out_dtype == torch.float32:
                 return torch.mm(x, w.t(), out_dtype=torch.float32)
             y = torch.nn.functional.linear(x, w, None if bias is None else bias.to(torch.bfloat16))
             return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
