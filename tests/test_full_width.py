@@ -160,3 +160,51 @@ def test_decode_steps_of_40_and_64_rows(model, dtype, captured):
         runner.cache.close(rc)
     runner.cache.check()
     print(f"{dtype}/{'graphs' if captured else 'eager'}: 40- and 64-row steps, worst {worst:.2e} of the logit scale")
+
+
+def test_captured_step_of_160_rows_replayed(model):
+    """160 single-token rows: every product of the step is a library call (more rows than the engine's own
+    product kernels take), inside a captured graph.  The graph is replayed four times, with kernel-by-kernel
+    work of the same runner and synchronisations between the replays; every replay must give exactly what a
+    second runner without graphs gives for the same step, and the last one the plain implementation's logits."""
+    from mini_inference_engine_amd.engine.batch import StepRow
+    dtype, n = "bfloat16", 160
+    lengths = [5 + (i * 7) % 12 for i in range(n)]
+    requests = [prompt_tokens(k + 4, 500 + i) for i, k in enumerate(lengths)]
+    pages = n * 2 + 8
+    runners = [make_runner(model, dtype, pages, max_rows=n + 1, max_step_tokens=2048) for _ in range(2)]
+    runners[0].capture_decode_graphs((n,))
+    caches = [[r.cache.open(i) for i in range(n)] for r in runners]
+    fed = [0] * n
+
+    def feed(counts, want_last):
+        outs = []
+        for r, rc in zip(runners, caches):
+            rows = []
+            for i, c in enumerate(counts):
+                assert r.cache.reserve(rc[i], fed[i], c)
+                rows.append(StepRow(rc[i], requests[i][fed[i]:fed[i] + c], fed[i], [c - 1] if want_last else []))
+            outs.append(r.forward_step(rows))
+        for i, c in enumerate(counts):
+            fed[i] += c
+        return outs
+
+    feed(lengths, False)                                       # the prompts: kernel by kernel in both runners
+    assert not runners[0].last_step_captured
+    for replay in range(4):
+        got, eager = feed([1] * n, True)
+        assert runners[0].last_step_captured and not runners[1].last_step_captured
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), f"replay {replay} of the captured step differs from the step launched kernel by kernel"
+        # work of another kind between the replays
+        scratch = runners[0].cache.open("between")
+        assert runners[0].cache.reserve(scratch, 0, 40)
+        runners[0].forward_step([StepRow(scratch, prompt_tokens(40, 900 + replay), 0, [39])])
+        runners[0].cache.close(scratch)
+        torch.cuda.synchronize()
+    worst = 0.0
+    for i in range(0, n, 16):
+        expect = plain_logits(model, dtype, requests[i])
+        worst = max(worst, worst_error(got[i][None], expect[fed[i] - 1:fed[i]], BF16_TOL, f"request {i}",
+                                       scale=float(expect.abs().max())))
+    print(f"160-row captured step: four replays equal the eager step; worst {worst:.2e} of the logit scale")

@@ -697,6 +697,19 @@ def test_prefill_attention_geometries(ops, geom, window):
     torch.testing.assert_close(out.float(), generic.float(), **ATT_TOL[dtype])
 
 
+@pytest.mark.parametrize("geom", [(32, 32, 16, 16), (32, 32, 128, 16), (64, 8, 64, 32)])
+def test_prefill_attention_many_workgroups(ops, geom):
+    """Rows and heads enough for the kernel's other way of spending eight waves (over twice the queries of a
+    workgroup instead of over two halves of the keys): the launcher picks it from the size of the grid."""
+    Hq, Hkv, D, page = geom
+    ctx = [700, 600, 650, 603]
+    qn = [600, 600, 600, 603]
+    dtype = torch.bfloat16
+    q, kc, vc, group, step = paged_setup(ctx, qn, Hq, Hkv, D, page, dtype, seed=D + Hkv)
+    out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1.1 / math.sqrt(D), None)
+    torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+
+
 def test_prefill_attention_ignores_stale_pages_bf16(ops):
     Hq, Hkv, D, page = 8, 2, 64, 16
     ctx, qn = [37, 5, 64, 130, 33], [30, 5, 2, 67, 33]
