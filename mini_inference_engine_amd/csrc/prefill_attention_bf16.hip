@@ -380,6 +380,7 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
       // The halves join: the second half's state goes through the LDS (item i of lane l at 4 (64 i + l), a
       // region a wave), the first half rescales both to the common maximum.  l and O are per-lane partial
       // sums, m is the same in a query's two lanes.
+      static_assert(KS == 1 || SUB_WAVES * 64 * (2 + 16 * DT32) * 4 <= 2 * KS * PF_BUF, "the halves' exchange must fit the buffers");
       float* xch = reinterpret_cast<float*>(pf_lds) + wsub * (64 * (2 + 16 * DT32)) + lane;
       __syncthreads();                                 // everybody is done with the keys and values
       if (wk == 1) {
