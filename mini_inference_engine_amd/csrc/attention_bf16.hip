@@ -20,15 +20,32 @@ constexpr int NW_SPLIT = D > 128 ? 2 : 4;    // waves per workgroup (bounded by 
 // has a whole context to read, and eight waves keep twice the loads in flight for it.
 constexpr int NW_WHOLE = D > 128 ? 2 : (D > 64 ? 4 : 8);
 
-template <int NW>
+// What the kernel needs to finish the q/k/v projection of its row itself (FROM_SUMS): the projection's
+// float32 sums, split over K or not, instead of q; the angle tables; where the row's new key and value go.
+// A workgroup then owns everything of its (row, kv head): it adds the splits up, rotates its group's q heads
+// (kept in the LDS) and its k head, writes k and v to their cache slot, and goes on as if another kernel had.
+// Only for unsplit contexts and groups of up to 16 heads (one workgroup per row and kv head).
+struct ProjectionSums {
+  const float* part;         // [splits, rows, ld]: q heads, k heads, v heads
+  int splits;
+  size_t split_stride;       // floats from one split to the next
+  long ld;
+  const float* cos_t;        // [positions, D / 2]
+  const float* sin_t;
+  const int* slots;          // [rows] cache slot of each row's token
+};
+
+template <int NW, bool FROM_SUMS>
 __global__ void __launch_bounds__(NW * 64)
-decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* __restrict__ k_cache,
-                        const bf16* __restrict__ v_cache, bf16* __restrict__ out, float* __restrict__ o_part,
+decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache, bf16* v_cache,
+                        bf16* __restrict__ out, float* __restrict__ o_part,
                         float* __restrict__ lse_part, const int* __restrict__ block_tables, int max_blocks,
                         const int* __restrict__ positions, int Hq, int Hkv, int head_tiles, int page,
-                        float scale_log2, int window, int partition, int num_splits) {
+                        float scale_log2, int window, int partition, int num_splits, ProjectionSums proj) {
   __shared__ float s_m[NW][16], s_l[NW][16], s_M[16], s_L[16];
   __shared__ float s_o[NW][16][D + 1];
+  __shared__ __align__(16) bf16 s_q[FROM_SUMS ? 16 : 1][D];
+  __shared__ __align__(16) bf16 s_k[FROM_SUMS ? D : 1], s_v[FROM_SUMS ? D : 1];   // the row's own new key and value
   const int b = blockIdx.x;
   const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
   const int s = blockIdx.z;
@@ -48,7 +65,7 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
   for (int ks = 0; ks < KS; ++ks) {
     const int d0 = ks * 32 + kb * 8;
     qf[ks].q = make_uint4(0, 0, 0, 0);
-    if (head_ok && d0 < D) qf[ks].q = *reinterpret_cast<const uint4*>(q + (size_t)b * q_stride + (size_t)head * D + d0);
+    if (!FROM_SUMS && head_ok && d0 < D) qf[ks].q = *reinterpret_cast<const uint4*>(q + (size_t)b * q_stride + (size_t)head * D + d0);
   }
   struct KeyBlock {
     Frag a[2][KS];      // keys: 16 keys x 32 dims each
@@ -88,6 +105,48 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
   if (AHEAD && window <= 0) load_block(b0, begin0 + BLOCK_KEYS * wave);
 
   const int pos = pos_raw;
+  if (FROM_SUMS) {
+    // the row's own q, k and v from the projection's sums (the expressions of the kernel that does this alone)
+    const int slot = proj.slots[b], half = D >> 1;
+    const float* pr = proj.part + (size_t)b * proj.ld;
+    const float* cr = proj.cos_t + (size_t)pos * half;
+    const float* sr = proj.sin_t + (size_t)pos * half;
+    bf16* kdst = k_cache + (((size_t)(slot / page) * Hkv + kvh) * page + (size_t)(slot % page)) * D;
+    for (int t = threadIdx.x; t < (G + 1) * half; t += NW * 64) {
+      const int hh = t / half, j = t - hh * half;
+      const float* src = pr + (size_t)(hh < G ? kvh * G + hh : Hq + kvh) * D + j;
+      float x1 = 0.f, x2 = 0.f;
+      add_splits(x1, src, proj.splits, proj.split_stride);
+      add_splits(x2, src + half, proj.splits, proj.split_stride);
+      const float c = cr[j], sn = sr[j];
+      float o1, o2;
+      rotate_pair(x1, x2, c, sn, o1, o2);
+      bf16* dst = hh < G ? s_q[hh] : s_k;
+      dst[j] = __float2bfloat16(o1);
+      dst[j + half] = __float2bfloat16(o2);
+      if (hh == G) {
+        kdst[j] = __float2bfloat16(o1);
+        kdst[j + half] = __float2bfloat16(o2);
+      }
+    }
+    bf16* vdst = v_cache + ((size_t)(slot / page) * Hkv + kvh) * page * D + (size_t)(slot % page);
+    for (int d = threadIdx.x; d < D; d += NW * 64) {
+      float v = 0.f;
+      add_splits(v, pr + (size_t)(Hq + Hkv + kvh) * D + d, proj.splits, proj.split_stride);
+      vdst[(size_t)d * page] = __float2bfloat16(v);
+      s_v[d] = __float2bfloat16(v);
+    }
+    // The waves meet over what went into the LDS only; the stores to the cache are not waited for, because
+    // nobody here reads them back: the block that holds the row's own key takes it from the LDS (compute()).
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 32 + kb * 8;
+      if (head_ok && d0 < D) qf[ks].q = *reinterpret_cast<const uint4*>(&s_q[g][d0]);
+    }
+  }
   const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
   const int begin = (lo & ~(BLOCK_KEYS - 1)) + s * partition;
   const int end = begin + partition < pos + 1 ? begin + partition : pos + 1;
@@ -104,6 +163,29 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* _
   for (int dt = 0; dt < DT; ++dt) O[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   auto compute = [&](KeyBlock& B, int blk) {
+    if (FROM_SUMS && pos >= blk && pos < blk + BLOCK_KEYS) {       // (the same for the whole wave)
+      // what was loaded for the row's own key is whatever its slot held: the key and value come from the LDS
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        if (blk + 16 * t + col == pos) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            const int d0 = ks * 32 + kb * 8;
+            B.a[t][ks].q = *reinterpret_cast<const uint4*>(&s_k[d0 < D ? d0 : 0]);
+          }
+        }
+#pragma unroll
+      for (int wi = 0; wi < 4; ++wi) {                           // word wi of a value fragment: two keys
+        const int key = blk + 16 * (wi >> 1) + 4 * kb + 2 * (wi & 1);
+        const bool low = key == pos, high = key + 1 == pos;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const uint32_t nv = (uint32_t)__bfloat16_as_ushort(s_v[dt * 16 + col]);
+          const uint32_t w = B.va[dt].w[wi];
+          B.va[dt].w[wi] = low ? (w & 0xFFFF0000u) | nv : (high ? (w & 0x0000FFFFu) | (nv << 16) : w);
+        }
+      }
+    }
     if (D % 32 != 0) {
       // the last 32-dim step of the keys is half empty: its upper lanes were loaded from dim 0
 #pragma unroll
@@ -314,19 +396,52 @@ MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_
   const int G = Hq / Hkv, head_tiles = (G + 15) / 16;
   if ((long)Hkv * head_tiles > 65535) MIE_FAIL("decode_attention: too many head tiles for the grid");
   dim3 grid(rows, Hkv * head_tiles, num_splits);
+  // (the kernel writes the caches only when it is given the projection's sums)
+  bf16* kc = (bf16*)const_cast<void*>(k_cache);
+  bf16* vc = (bf16*)const_cast<void*>(v_cache);
   if (num_splits == 1 && NW_WHOLE != NW_SPLIT)
-    hipLaunchKernelGGL(decode_attention_kernel<NW_WHOLE>, grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)q, q_stride,
-                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, o_part, lse_part, block_tables, max_blocks,
-                       positions, Hq, Hkv, head_tiles, page, scale * 1.4426950408889634f, window, partition, num_splits);
+    hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, false>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)q, q_stride,
+                       kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
+                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{});
   else
-    hipLaunchKernelGGL(decode_attention_kernel<NW_SPLIT>, grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)q, q_stride,
-                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, o_part, lse_part, block_tables, max_blocks,
-                       positions, Hq, Hkv, head_tiles, page, scale * 1.4426950408889634f, window, partition, num_splits);
+    hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, false>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)q, q_stride,
+                       kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
+                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{});
   MIE_CHECK_LAUNCH("decode_attention");
   if (num_splits > 1) {
     hipLaunchKernelGGL(merge_splits_kernel, dim3(rows * Hq), dim3(64), 0, stream, o_part, lse_part, (bf16*)out, num_splits);
     MIE_CHECK_LAUNCH("merge_splits");
   }
+  return 0;
+}
+
+
+// The q/k/v projection's end and the attention in one kernel, for steps whose rows and kv heads alone fill
+// the GPU (contexts unsplit).  part [splits, rows, ld] float32: the projection's sums (q heads, k heads, v
+// heads), to be added up in split order; rotary over the whole head with angles from cos / sin [positions,
+// D / 2]; the row's k and v go to cache slot slots[row], which must be the slot of key positions[row] in the
+// row's block table.  Groups of up to 16 query heads a kv head.  partition as for mie_decode_attention (at least the
+// longest context).
+MIE_EXPORT int mie_decode_attention_from_sums(const float* part, int splits, long split_stride, long ld, const float* cos_t,
+                                              const float* sin_t, const int* slots, void* k_cache, void* v_cache, void* out,
+                                              const int* block_tables, int max_blocks, const int* positions, int rows, int Hq,
+                                              int Hkv, int head_dim, int page, float scale, int window, int partition,
+                                              hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (head_dim != D) MIE_FAIL("decode_attention_from_sums: built for head_dim %d, called with %d", D, head_dim);
+  if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("decode_attention_from_sums: %d query heads on %d kv heads", Hq, Hkv);
+  if (Hq / Hkv > 16) MIE_FAIL("decode_attention_from_sums: groups of %d query heads (at most 16)", Hq / Hkv);
+  if (page < 16 || page % 16) MIE_FAIL("decode_attention_from_sums: page size %d (multiples of 16)", page);
+  if (partition <= 0 || partition % (BLOCK_KEYS * NW_SPLIT)) MIE_FAIL("decode_attention_from_sums: partition %d is no multiple of %d", partition, BLOCK_KEYS * NW_SPLIT);
+  if (!part || !cos_t || !sin_t || !slots || !k_cache || !v_cache || !out || !positions || !block_tables) MIE_FAIL("decode_attention_from_sums: null operand");
+  if (splits < 1 || ld < (long)(Hq + 2 * Hkv) * D || (splits > 1 && split_stride < (long)rows * ld)) MIE_FAIL("decode_attention_from_sums: %d splits, stride %ld, row stride %ld", splits, split_stride, ld);
+  if (max_blocks <= 0 || Hkv > 65535) MIE_FAIL("decode_attention_from_sums: max_blocks %d, %d kv heads", max_blocks, Hkv);
+  const ProjectionSums proj = {part, splits, (size_t)split_stride, ld, cos_t, sin_t, slots};
+  dim3 grid(rows, Hkv, 1);
+  hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, true>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)nullptr, 0L,
+                     (bf16*)k_cache, (bf16*)v_cache, (bf16*)out, (float*)nullptr, (float*)nullptr, block_tables, max_blocks, positions,
+                     Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj);
+  MIE_CHECK_LAUNCH("decode_attention_from_sums");
   return 0;
 }
 

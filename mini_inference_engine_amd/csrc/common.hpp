@@ -50,6 +50,31 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return t;
 }
 
+// ---- partial sums of a product whose K was split over workgroups
+constexpr int MIE_SPLITS_AHEAD = 8;      // splits whose loads are issued together
+
+// acc += the splits' values at p, in split order.  The loads of up to MIE_SPLITS_AHEAD splits are issued
+// together, each unconditional from an address clamped to the last split (what it brings for a split that does
+// not exist is not added), so a kernel waits for memory once per MIE_SPLITS_AHEAD splits and not once per split.
+template <typename V>
+__device__ __forceinline__ void add_splits(V& acc, const V* p, int splits, size_t split_stride_v) {
+  for (int s0 = 0; s0 < splits; s0 += MIE_SPLITS_AHEAD) {
+    V v[MIE_SPLITS_AHEAD];
+#pragma unroll
+    for (int j = 0; j < MIE_SPLITS_AHEAD; ++j) v[j] = p[(size_t)(s0 + j < splits ? s0 + j : splits - 1) * split_stride_v];
+#pragma unroll
+    for (int j = 0; j < MIE_SPLITS_AHEAD; ++j)
+      if (s0 + j < splits) acc += v[j];
+  }
+}
+
+// ---- rotary position encoding of one pair, from float32: (x1, x2) turned by the angle whose cosine and sine
+// are c and s.  One spelling for every kernel that rotates float32 sums, so that they round alike.
+__device__ __forceinline__ void rotate_pair(float x1, float x2, float c, float s, float& o1, float& o2) {
+  o1 = fmaf(x1, c, -(x2 * s));
+  o2 = fmaf(x2, c, x1 * s);
+}
+
 // ---- host-side error plumbing
 static thread_local char g_mie_error[512];
 #define MIE_FAIL(...)                                        \

@@ -158,28 +158,12 @@ mid_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict__ W
 enum { RED_STORE_BF16 = 0, RED_STORE_F32 = 1, RED_ADD = 2, RED_ADD_NORM = 3 };
 constexpr int RED_THREADS = 512;
 constexpr int RED_VEC = 4;        // float4 a thread: rows up to 8192 wide
-constexpr int RED_AHEAD = 8;      // splits whose loads are issued together
 
 __device__ __forceinline__ void store_bf16x4(bf16* p, float4 v) {
   uint2 u;
   u.x = (uint32_t)__bfloat16_as_ushort(__float2bfloat16(v.x)) | ((uint32_t)__bfloat16_as_ushort(__float2bfloat16(v.y)) << 16);
   u.y = (uint32_t)__bfloat16_as_ushort(__float2bfloat16(v.z)) | ((uint32_t)__bfloat16_as_ushort(__float2bfloat16(v.w)) << 16);
   *reinterpret_cast<uint2*>(p) = u;
-}
-
-// acc += the splits' values at p, in split order.  The loads of up to RED_AHEAD splits are issued together,
-// each unconditional from an address clamped to the last split (what it brings for a split that does not
-// exist is not added), so the kernel waits for memory once per RED_AHEAD splits and not once per split.
-template <typename V>
-__device__ __forceinline__ void add_splits(V& acc, const V* p, int splits, size_t split_stride_v) {
-  for (int s0 = 0; s0 < splits; s0 += RED_AHEAD) {
-    V v[RED_AHEAD];
-#pragma unroll
-    for (int j = 0; j < RED_AHEAD; ++j) v[j] = p[(size_t)(s0 + j < splits ? s0 + j : splits - 1) * split_stride_v];
-#pragma unroll
-    for (int j = 0; j < RED_AHEAD; ++j)
-      if (s0 + j < splits) acc += v[j];
-  }
 }
 
 // One workgroup a row; N a multiple of 4, at most 4 * RED_THREADS * RED_VEC.  y = sum of the splits in
@@ -263,8 +247,10 @@ reduce_rope_kv_kernel(const float* __restrict__ part, int splits, size_t split_s
       float x1 = 0.f, x2 = 0.f;
       add_splits(x1, pr + j, splits, split_stride);
       add_splits(x2, pr + j + half, splits, split_stride);
-      dst[j] = __float2bfloat16(x1 * c - x2 * sn);
-      dst[j + half] = __float2bfloat16(x2 * c + x1 * sn);
+      float o1, o2;
+      rotate_pair(x1, x2, c, sn, o1, o2);
+      dst[j] = __float2bfloat16(o1);
+      dst[j + half] = __float2bfloat16(o2);
     }
   } else {
     bf16* dst = v_cache + ((size_t)(slot / page) * Hkv + (head - Hq - Hkv)) * page * D + (size_t)(slot % page);

@@ -163,11 +163,16 @@ rotary_kv_store_sums_kernel(const float* __restrict__ sums, long ld, bf16* __res
     const float4 a = *reinterpret_cast<const float4*>(src + j), b = *reinterpret_cast<const float4*>(src + j + half);
     const float4 c = *reinterpret_cast<const float4*>(cos_t + (size_t)s_pos[i] * half + j);
     const float4 sn = *reinterpret_cast<const float4*>(sin_t + (size_t)s_pos[i] * half + j);
+    float r1[4], r2[4];
+    rotate_pair(a.x, b.x, c.x, sn.x, r1[0], r2[0]);
+    rotate_pair(a.y, b.y, c.y, sn.y, r1[1], r2[1]);
+    rotate_pair(a.z, b.z, c.z, sn.z, r1[2], r2[2]);
+    rotate_pair(a.w, b.w, c.w, sn.w, r1[3], r2[3]);
     uint2 o1, o2;
-    o1.x = rs_pack(a.x * c.x - b.x * sn.x, a.y * c.y - b.y * sn.y);
-    o1.y = rs_pack(a.z * c.z - b.z * sn.z, a.w * c.w - b.w * sn.w);
-    o2.x = rs_pack(b.x * c.x + a.x * sn.x, b.y * c.y + a.y * sn.y);
-    o2.y = rs_pack(b.z * c.z + a.z * sn.z, b.w * c.w + a.w * sn.w);
+    o1.x = rs_pack(r1[0], r1[1]);
+    o1.y = rs_pack(r1[2], r1[3]);
+    o2.x = rs_pack(r2[0], r2[1]);
+    o2.y = rs_pack(r2[2], r2[3]);
     bf16* dst;
     if (head < Hq) {
       dst = q_out + (size_t)t * ldq + (size_t)head * D;

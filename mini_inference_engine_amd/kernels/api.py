@@ -88,10 +88,12 @@ class KernelBackend:
         raise NotImplementedError
 
     def linear_rotary_kv_store(self, x, w_qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
-                               k_cache, v_cache, slot_mapping):
+                               k_cache, v_cache, slot_mapping, for_attention: bool = False):
         """The fused q/k/v projection followed by rotary_kv_store.  Returns a tensor whose first
         Hq * D columns are the encoded q (the whole qkv, or q alone): a backend may do all of it in
-        one kernel.  ``x`` is a tensor or a Normed."""
+        one kernel.  ``x`` is a tensor or a Normed.  ``for_attention``: the caller hands the result to this
+        backend's ``paged_attention`` of the same step over the same caches, and to nothing else; a backend
+        may then return an object of its own that only that call understands (work it has put off)."""
         qkv = self.linear(x, w_qkv)
         self.rotary_kv_store(qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim, k_cache,
                              v_cache, slot_mapping)

@@ -39,6 +39,35 @@ def _rows_ok(t: torch.Tensor, what: str) -> None:
                          f"strides {t.stride()}")
 
 
+class ProjectionSums:
+    """The q/k/v projection of a step as float32 sums [splits, tokens, (Hq + 2 Hkv) D], not yet added up, rotated
+    or written to the cache (operands checked).  ``finish()`` does that in a kernel of its own and gives q
+    [tokens, Hq * D]; ``paged_attention`` lets its decode kernel do it instead where that kernel has a workgroup
+    of its own for every row and kv head."""
+
+    def __init__(self, ops, part, positions, cos, sin, slots, k_cache, v_cache, Hq, Hkv, D, page):
+        self.ops, self.part, self.positions, self.cos, self.sin, self.slots = ops, part, positions, cos, sin, slots
+        self.k_cache, self.v_cache, self.Hq, self.Hkv, self.D, self.page = k_cache, v_cache, Hq, Hkv, D, page
+
+    def finish(self):
+        ops, part = self.ops, self.part
+        splits, M, _ = part.shape
+        q = torch.empty((M, self.Hq * self.D), dtype=torch.bfloat16, device=part.device)
+        if splits == 1 and M > HipBackend.MID_MAX_ROWS:
+            lib = ops.lib("rope_kv")
+            library.check(lib, lib.mie_rotary_kv_store_sums(
+                _ptr(part), part.stride(1), _ptr(q), q.stride(0), _ptr(self.positions), _ptr(self.cos), _ptr(self.sin),
+                _ptr(self.slots), _ptr(self.k_cache), _ptr(self.v_cache), self.Hq, self.Hkv, self.D, self.page, M,
+                ops._stream()))
+        else:
+            lib = ops.lib("gemm_mid_bf16")
+            library.check(lib, lib.mie_mid_reduce_rope_kv(
+                _ptr(part), splits, M, _ptr(q), q.stride(0), _ptr(self.positions), _ptr(self.cos), _ptr(self.sin),
+                _ptr(self.slots), _ptr(self.k_cache), _ptr(self.v_cache), self.Hq, self.Hkv, self.D, self.page,
+                ops._stream()))
+        return q
+
+
 class HipBackend(KernelBackend):
     name = "hip-gfx950"
 
@@ -306,7 +335,7 @@ class HipBackend(KernelBackend):
         return self.silu_mul(self.linear(x, w_gate_up), intermediate)
 
     def linear_rotary_kv_store(self, x, w_qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
-                               k_cache, v_cache, slot_mapping):
+                               k_cache, v_cache, slot_mapping, for_attention: bool = False):
         Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
         can_rope = (Hkv > 0 and rotary_dim == D and D % 16 == 0 and k_cache is not None
                     and k_cache.dtype == torch.bfloat16)
@@ -318,7 +347,8 @@ class HipBackend(KernelBackend):
             x = x.materialize()
         fused = can_rope and self._skinny_ok(x, w_qkv, None)
         if not fused and can_rope and self._mid_ok(x, w_qkv, None) and self.act_dtype == torch.bfloat16:
-            return self._mid_rotary_kv_store(x, w_qkv, positions, cos, sin, Hq, Hkv, D, k_cache, v_cache, slot_mapping)
+            return self._mid_rotary_kv_store(x, w_qkv, positions, cos, sin, Hq, Hkv, D, k_cache, v_cache, slot_mapping,
+                                             for_attention)
         if (not fused and can_rope and not self.true_fp32 and self.act_dtype == torch.bfloat16
                 and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16):
             # many rows: library product with float32 sums, then rotary and cache write from those sums (q and k
@@ -329,12 +359,8 @@ class HipBackend(KernelBackend):
             page = self._check_rope_operands("linear_rotary_kv_store", M, K, w_qkv, positions, cos, sin, Hq, Hkv, D,
                                              k_cache, v_cache, slot_mapping)
             sums = torch.mm(x, w_qkv.t(), out_dtype=torch.float32)
-            q = torch.empty((M, Hq * D), dtype=torch.bfloat16, device=x.device)
-            lib = self.lib("rope_kv")
-            library.check(lib, lib.mie_rotary_kv_store_sums(
-                _ptr(sums), sums.stride(0), _ptr(q), q.stride(0), _ptr(positions), _ptr(cos), _ptr(sin),
-                _ptr(slot_mapping), _ptr(k_cache), _ptr(v_cache), Hq, Hkv, D, page, M, self._stream()))
-            return q
+            pending = ProjectionSums(self, sums[None], positions, cos, sin, slot_mapping, k_cache, v_cache, Hq, Hkv, D, page)
+            return pending if for_attention else pending.finish()
         if not fused:
             return super().linear_rotary_kv_store(x, w_qkv, positions, cos, sin, rotary_dim, Hq, Hkv, D, k_cache,
                                                   v_cache, slot_mapping)
@@ -367,20 +393,18 @@ class HipBackend(KernelBackend):
                 raise ValueError(f"{what}: {name} must be contiguous int32 [{M}]")
         return page
 
-    def _mid_rotary_kv_store(self, x, w_qkv, positions, cos, sin, Hq, Hkv, D, k_cache, v_cache, slot_mapping):
+    def _mid_rotary_kv_store(self, x, w_qkv, positions, cos, sin, Hq, Hkv, D, k_cache, v_cache, slot_mapping,
+                             for_attention=False):
         """The q/k/v projection of 33 to 128 rows: split product, then one kernel that adds the partial
-        results, rotates q and k and writes k and v to the cache.  Returns q [M, Hq * D]."""
+        results, rotates q and k and writes k and v to the cache.  Returns q [M, Hq * D] (for_attention: the
+        partial results, for paged_attention to finish)."""
         self._on_device(x, w_qkv, positions, cos, sin, k_cache, v_cache, slot_mapping)
         M, K = x.shape
         page = self._check_rope_operands("linear_rotary_kv_store", M, K, w_qkv, positions, cos, sin, Hq, Hkv, D,
                                          k_cache, v_cache, slot_mapping)
-        part = self._mid_partials(x, w_qkv)
-        q = torch.empty((M, Hq * D), dtype=torch.bfloat16, device=x.device)
-        lib = self.lib("gemm_mid_bf16")
-        library.check(lib, lib.mie_mid_reduce_rope_kv(
-            _ptr(part), part.shape[0], M, _ptr(q), q.stride(0), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
-            _ptr(k_cache), _ptr(v_cache), Hq, Hkv, D, page, self._stream()))
-        return q
+        pending = ProjectionSums(self, self._mid_partials(x, w_qkv), positions, cos, sin, slot_mapping, k_cache, v_cache,
+                                 Hq, Hkv, D, page)
+        return pending if for_attention else pending.finish()
 
     def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
                         k_cache, v_cache, slot_mapping):
@@ -413,15 +437,16 @@ class HipBackend(KernelBackend):
 
     def _check_attention(self, qkv, Hq, Hkv, D, k_cache, v_cache, group, step):
         _rows_ok(qkv, "paged_attention: qkv")
-        T = qkv.shape[0]
         if qkv.shape[1] < Hq * D:
             raise ValueError(f"paged_attention: qkv has {qkv.shape[1]} columns, fewer than {Hq * D}")
+        return self._check_attention_cache(qkv.shape[0], qkv.dtype, Hkv, D, k_cache, v_cache, group, step)
+
+    def _check_attention_cache(self, T, dtype, Hkv, D, k_cache, v_cache, group, step):
         pages, hk, page, d = k_cache.shape
         if (hk, d) != (Hkv, D) or tuple(v_cache.shape) != (pages, Hkv, D, page):
             raise ValueError(f"paged_attention: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for "
                              f"{Hkv} kv heads of {D}")
-        if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype or not (k_cache.is_contiguous() and
-                                                                            v_cache.is_contiguous()):
+        if k_cache.dtype != dtype or v_cache.dtype != dtype or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
             raise ValueError("paged_attention: caches must be contiguous and of the activation dtype")
         bt = group.block_tables
         if bt.dtype != torch.int32 or bt.dim() != 2 or bt.stride(1) != 1 or bt.stride(0) != bt.shape[1]:
@@ -454,10 +479,38 @@ class HipBackend(KernelBackend):
         partition = -(-(-(-context_bound // splits)) // block_keys) * block_keys
         return partition, max(1, -(-context_bound // partition))
 
+    def _decode_attention_from_sums(self, pending, Hq, Hkv, D, k_cache, v_cache, group, step, scale, window, forced):
+        """A step of single-token rows whose rows and kv heads alone fill the GPU: the decode kernel finishes the
+        projection itself (no kernel between product and attention).  None: not such a step."""
+        T = pending.part.shape[1]
+        if (forced or step.num_decode_rows != T or step.num_tokens != T or Hq // Hkv > 16
+                or pending.k_cache is not k_cache or pending.v_cache is not v_cache):
+            return None
+        lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))
+        block_keys = lib.mie_decode_block_keys()
+        partition, splits = self.decode_splits(T, Hq, Hkv, step.max_context, window, block_keys)
+        if splits != 1:
+            return None
+        part = pending.part
+        self._on_device(k_cache, v_cache)
+        _, _, bt = self._check_attention_cache(T, torch.bfloat16, Hkv, D, k_cache, v_cache, group, step)
+        out = torch.empty((T, Hq * D), dtype=torch.bfloat16, device=part.device)
+        library.check(lib, lib.mie_decode_attention_from_sums(
+            _ptr(part), part.shape[0], part.stride(0), part.stride(1), _ptr(pending.cos), _ptr(pending.sin),
+            _ptr(pending.slots), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(bt), bt.shape[1], _ptr(step.positions), T,
+            Hq, Hkv, D, pending.page, float(scale), int(window or 0), partition, self._stream()))
+        return out
+
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
                         window, force_generic: bool = False, num_splits: int | None = None):
-        self._on_device(qkv, k_cache, v_cache)
         Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
+        if isinstance(qkv, ProjectionSums):
+            out = self._decode_attention_from_sums(qkv, Hq, Hkv, D, k_cache, v_cache, group, step, scale, window,
+                                                   force_generic or num_splits is not None)
+            if out is not None:
+                return out
+            qkv = qkv.finish()
+        self._on_device(qkv, k_cache, v_cache)
         T, page, bt = self._check_attention(qkv, Hq, Hkv, D, k_cache, v_cache, group, step)
         out = torch.empty((T, Hq * D), dtype=qkv.dtype, device=qkv.device)
         done = 0

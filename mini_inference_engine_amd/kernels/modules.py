@@ -41,6 +41,7 @@ register_kernel_module("gemm_mid_bf16", {
 })
 register_kernel_module("attention_bf16", {
     "mie_decode_attention": [P, L, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P],
+    "mie_decode_attention_from_sums": [P, I, L, L, P, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, P],
     "mie_decode_attention_static": [P, L, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P],
     "mie_decode_attention_static_setup": [],
     "mie_decode_block_keys": [],

@@ -47,10 +47,11 @@ class RotaryHalfSplit(PositionEncoding):
                             num_kv_heads, self.head_dim, k_cache, v_cache, slots)
 
     def project_encode_store(self, ops, x, w_qkv, step, num_q_heads, num_kv_heads, k_cache, v_cache, slots):
-        """Projection, encoding and cache write together; returns a tensor whose first Hq * D columns
-        are the encoded q.  The backend may run it as one kernel."""
+        """Projection, encoding and cache write together; returns what the backend's paged_attention takes as
+        its ``qkv`` (a tensor whose first Hq * D columns are the encoded q, or work the backend has put off
+        until then).  The backend may run it as one kernel."""
         return ops.linear_rotary_kv_store(x, w_qkv, step.positions, self.cos, self.sin, self.rotary_dim, num_q_heads,
-                                          num_kv_heads, self.head_dim, k_cache, v_cache, slots)
+                                          num_kv_heads, self.head_dim, k_cache, v_cache, slots, for_attention=True)
 
 
 @register_position_encoding("none")
@@ -66,4 +67,4 @@ class NoPosition(PositionEncoding):
 
     def project_encode_store(self, ops, x, w_qkv, step, num_q_heads, num_kv_heads, k_cache, v_cache, slots):
         return ops.linear_rotary_kv_store(x, w_qkv, step.positions, None, None, 0, num_q_heads, num_kv_heads,
-                                          self.head_dim, k_cache, v_cache, slots)
+                                          self.head_dim, k_cache, v_cache, slots, for_attention=True)

@@ -562,6 +562,60 @@ def test_decode_attention_split_count_and_static_bound(ops, ctx, splits):
     torch.testing.assert_close(out2.double(), expect, **ATT_TOL[dtype])
 
 
+@pytest.mark.parametrize("geom", [(32, 4, 64, 16, 64), (8, 8, 128, 16, 40), (6, 2, 32, 32, 130), (16, 1, 16, 16, 257),
+                                  (10, 5, 48, 16, 52), (4, 4, 256, 16, 64)])
+@pytest.mark.parametrize("window", [None, 40])
+def test_decode_attention_finishes_the_projection(engine_ops, geom, window):
+    """Steps of single-token rows whose rows x kv heads are 256 workgroups or more: the decode kernel takes the
+    q/k/v projection's float32 sums (partial sums of the split product up to 128 rows, the library's sums above)
+    and does rotary, cache write and attention itself.  Against the same step done by the kernels that are each
+    checked against their references elsewhere: sum + rotary + cache write, then attention over the cache.
+    Contexts of 1 key, around the kernel's first blocks (which it asks for before the new key is written),
+    at page edges, and long ones."""
+    from mini_inference_engine_amd.kernels.hip_backend import ProjectionSums
+    from mini_inference_engine_amd.parts.rope import rotary_tables
+    Hq, Hkv, D, page, M = geom
+    o = engine_ops
+    assert M * Hkv >= o.DECODE_WHOLE_WORKGROUPS
+    ctx = [1, 2, 16, 17, 31, 32, 33, 64, 65, 127, 128, 129, 255, 256, 257, 300, 1000, 48]
+    ctx = (ctx * (M // len(ctx) + 1))[:M]
+    K = 264
+    torch.manual_seed(D + M)
+    _, kc, vc, group, step = paged_setup(ctx, [1] * M, Hq, Hkv, D, page, torch.bfloat16, seed=D + Hkv)
+    cos, sin = (t.to(DEV) for t in rotary_tables(10000.0, D, max(ctx) + 1))
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn((Hq + 2 * Hkv) * D, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    pos = step.positions
+    bt = group.block_tables
+    slots = (bt[torch.arange(M, device=DEV), (pos // page).long()] * page + pos % page).to(torch.int32)
+    scale = 0.9 / math.sqrt(D)
+
+    kc1, vc1 = kc.clone(), vc.clone()
+    pending = o.linear_rotary_kv_store(x, w, pos, cos, sin, D, Hq, Hkv, D, kc1, vc1, slots, for_attention=True)
+    assert isinstance(pending, ProjectionSums), "this many rows must leave the projection unfinished"
+    assert torch.equal(kc1, kc) and torch.equal(vc1, vc), "nothing is written before the attention runs"
+    out1 = o.paged_attention(pending, Hq, Hkv, D, kc1, vc1, group, step, scale, window)
+
+    kc2, vc2 = kc.clone(), vc.clone()
+    q2 = o.linear_rotary_kv_store(x, w, pos, cos, sin, D, Hq, Hkv, D, kc2, vc2, slots)
+    assert torch.is_tensor(q2)
+    out2 = o.paged_attention(q2, Hq, Hkv, D, kc2, vc2, group, step, scale, window)
+    # the same sums in the same order, the same expressions: the new keys and values are the same numbers
+    assert torch.equal(vc1, vc2), f"{int((vc1 != vc2).sum())} values differ, by up to {float((vc1.float() - vc2.float()).abs().max())}"
+    assert torch.equal(kc1, kc2), f"{int((kc1 != kc2).sum())} keys differ, by up to {float((kc1.float() - kc2.float()).abs().max())}"
+    assert not torch.equal(kc1, kc), "the step's keys were written"
+    torch.testing.assert_close(out1.float(), out2.float(), atol=2e-3, rtol=2e-3)
+    # and against the exact attention over that cache
+    expect = ref.ref_paged_attention(q2, Hq, Hkv, D, kc2, vc2, bt, step.token_row, pos, scale, window, torch.float64)
+    torch.testing.assert_close(out1.double(), expect, **ATT_TOL[torch.bfloat16])
+    # a step that is not of this kind finishes the projection in a kernel of its own
+    kc3, vc3 = kc.clone(), vc.clone()
+    pending = o.linear_rotary_kv_store(x, w, pos, cos, sin, D, Hq, Hkv, D, kc3, vc3, slots, for_attention=True)
+    out3 = o.paged_attention(pending, Hq, Hkv, D, kc3, vc3, group, step, scale, window, num_splits=2)
+    assert torch.equal(kc3, kc2) and torch.equal(vc3, vc2)
+    torch.testing.assert_close(out3.double(), expect, **ATT_TOL[torch.bfloat16])
+
+
 @pytest.mark.parametrize("geom", [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 16), (40, 2, 80, 32), (8, 1, 128, 64),
                                   (2, 2, 256, 16), (12, 4, 96, 48), (17, 1, 64, 16)])
 @pytest.mark.parametrize("window", [None, 40])
