@@ -53,7 +53,7 @@ class ProjectionSums:
         ops, part = self.ops, self.part
         splits, M, _ = part.shape
         q = torch.empty((M, self.Hq * self.D), dtype=torch.bfloat16, device=part.device)
-        if splits == 1 and M > HipBackend.MID_MAX_ROWS:
+        if splits == 1:
             lib = ops.lib("rope_kv")
             library.check(lib, lib.mie_rotary_kv_store_sums(
                 _ptr(part), part.stride(1), _ptr(q), q.stride(0), _ptr(self.positions), _ptr(self.cos), _ptr(self.sin),

@@ -241,12 +241,13 @@ def test_mid_linear_refuses_what_it_cannot_run(engine_ops):
 @pytest.mark.parametrize("geom", [(2, 1, 16), (3, 1, 32), (4, 2, 48), (32, 4, 64), (5, 5, 96), (8, 2, 128), (2, 1, 256)])
 @pytest.mark.parametrize("M", [40, 64])
 def test_mid_projection_rotary_store(engine_ops, geom, M):
-    """Split projection, then one kernel for sum + rotary + cache write, against the separate references."""
+    """Split projection, then one kernel for sum + rotary + cache write, against the separate references
+    (K long enough for four splits at 40 rows, one split at 64)."""
     from mini_inference_engine_amd.parts.rope import rotary_tables
     Hq, Hkv, D = geom
     o = engine_ops
     torch.manual_seed(D + M)
-    K, page, pages = 264, 16, 12
+    K, page, pages = (1032 if M == 40 else 264), 16, 12
     cos, sin = (t.to(DEV) for t in rotary_tables(10000.0, D, 300))
     x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
     w = (torch.randn((Hq + 2 * Hkv) * D, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
@@ -579,7 +580,7 @@ def test_decode_attention_finishes_the_projection(engine_ops, geom, window):
     assert M * Hkv >= o.DECODE_WHOLE_WORKGROUPS
     ctx = [1, 2, 16, 17, 31, 32, 33, 64, 65, 127, 128, 129, 255, 256, 257, 300, 1000, 48]
     ctx = (ctx * (M // len(ctx) + 1))[:M]
-    K = 264
+    K = 1032 if window else 264          # four splits of K or one (where the product splits at all)
     torch.manual_seed(D + M)
     _, kc, vc, group, step = paged_setup(ctx, [1] * M, Hq, Hkv, D, page, torch.bfloat16, seed=D + Hkv)
     cos, sin = (t.to(DEV) for t in rotary_tables(10000.0, D, max(ctx) + 1))
