@@ -255,6 +255,17 @@ def measure_kernels(cfg, args) -> int:
     group = SimpleNamespace(block_tables=bt, max_blocks=bt.shape[1])
     t = timed(lambda i: ops.paged_attention(qkv, Hq, Hkv, D, kc, vc, group, step, D ** -0.5, None), 8)
     report(f"decode attention + merge, {M} rows of {ctx} keys", t, 2 * 2 * M * ctx * Hkv * D)
+    # ---- the q/k/v projection and the attention as the engine runs them in a step of M single-token rows
+    # (from 33 rows on the attention kernel may finish the projection itself)
+    w = weights(n_qkv, h)
+
+    def projection_and_attention(i):
+        pending = ops.linear_rotary_kv_store(x, w[i % copies], pos, cos, sin, D, Hq, Hkv, D, kc, vc, slots, for_attention=True)
+        ops.paged_attention(pending, Hq, Hkv, D, kc, vc, group, step, D ** -0.5, None)
+    t = timed(projection_and_attention, copies)
+    report(f"qkv product + rotary + cache write + decode attention, {M} rows of {ctx} keys", t,
+           2 * n_qkv * h + 2 * M * h + 2 * 2 * M * ctx * Hkv * D)
+    del w
     # ---- prefill: attention over a T-token prompt, and the library product it sits between
     qkv = torch.randn(T, n_qkv, device=dev).to(torch.bfloat16)
     pstep = SimpleNamespace(token_row=torch.zeros(T, device=dev, dtype=torch.int32),
