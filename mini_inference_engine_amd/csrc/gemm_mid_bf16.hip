@@ -36,34 +36,56 @@ constexpr int FRAG_BYTES = 1024;  // one operand fragment: 64 lanes x 16 bytes
 // wait until at most n vector memory loads of this wave are still on their way
 #define MID_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
 
-template <int OFF>
-__device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
-  u32x4 v;
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
-  return v;
-}
-// the reads above are done; the "+v" ties keep the compiler from using the registers before this point
-template <int MT>
-__device__ __forceinline__ void lds_wait(u32x4& w, u32x4 (&x)[MT]);
-template <>
-__device__ __forceinline__ void lds_wait<4>(u32x4& w, u32x4 (&x)[4]) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(w), "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]));
-}
-template <>
-__device__ __forceinline__ void lds_wait<8>(u32x4& w, u32x4 (&x)[8]) {
-  asm volatile("s_waitcnt lgkmcnt(0)"
-               : "+v"(w), "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]));
-}
+// The fragments of one k-step out of the LDS: the wave's weight fragment (at wbase) and the x fragments of all
+// row tiles (1 KB apart from xbase), read and waited for in one piece of assembly.  The compiler knows nothing
+// of the loads that write the LDS, so a read of the LDS it could see would make it wait for every load on its
+// way; and it must never see a register whose value is still to arrive (it may move it), so the wait is part
+// of the same piece.  OFF: byte offset of the k-step within the stage, XOFF: of its first x fragment.
+template <int MT, int OFF, int XOFF>
+struct LdsFragments;
+template <int OFF, int XOFF>
+struct LdsFragments<4, OFF, XOFF> {
+  static __device__ __forceinline__ void read(uint32_t wbase, uint32_t xbase, u32x4& w, u32x4 (&x)[4]) {
+    asm volatile(
+      "ds_read_b128 %0, %5 offset:%7\n\t"
+      "ds_read_b128 %1, %6 offset:%8\n\t"
+      "ds_read_b128 %2, %6 offset:%8+1024\n\t"
+      "ds_read_b128 %3, %6 offset:%8+2048\n\t"
+      "ds_read_b128 %4, %6 offset:%8+3072\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(w), "=&v"(x[0]), "=&v"(x[1]), "=&v"(x[2]), "=&v"(x[3])
+      : "v"(wbase), "v"(xbase), "n"(OFF), "n"(XOFF)
+      : "memory");
+  }
+};
+template <int OFF, int XOFF>
+struct LdsFragments<8, OFF, XOFF> {
+  static __device__ __forceinline__ void read(uint32_t wbase, uint32_t xbase, u32x4& w, u32x4 (&x)[8]) {
+    asm volatile(
+      "ds_read_b128 %0, %9 offset:%11\n\t"
+      "ds_read_b128 %1, %10 offset:%12\n\t"
+      "ds_read_b128 %2, %10 offset:%12+1024\n\t"
+      "ds_read_b128 %3, %10 offset:%12+2048\n\t"
+      "ds_read_b128 %4, %10 offset:%12+3072\n\t"
+      "ds_read_b128 %5, %10 offset:%12+4096\n\t"
+      "ds_read_b128 %6, %10 offset:%12+5120\n\t"
+      "ds_read_b128 %7, %10 offset:%12+6144\n\t"
+      "ds_read_b128 %8, %10 offset:%12+7168\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(w), "=&v"(x[0]), "=&v"(x[1]), "=&v"(x[2]), "=&v"(x[3]), "=&v"(x[4]), "=&v"(x[5]), "=&v"(x[6]), "=&v"(x[7])
+      : "v"(wbase), "v"(xbase), "n"(OFF), "n"(XOFF)
+      : "memory");
+  }
+};
 
 // One stage = KC k-steps; a k-step holds the waves' weight fragments, then the x fragments of the row tiles.
 template <int MT, int kc>
 struct StageReader {
   static constexpr int SF = MID_WAVES + MT;
+  static_assert(FRAG_BYTES == 1024, "the offsets in LdsFragments");
   static __device__ __forceinline__ void run(uint32_t base, uint32_t wbase, f32x4 (&acc)[MT]) {
     u32x4 w, x[MT];
-    w = lds_read16<kc * SF * FRAG_BYTES>(wbase);
-    read_x<0>(base, x);
-    lds_wait<MT>(w, x);
+    LdsFragments<MT, kc * SF * FRAG_BYTES, (kc * SF + MID_WAVES) * FRAG_BYTES>::read(wbase, base, w, x);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       Frag a, b;
@@ -72,11 +94,6 @@ struct StageReader {
       acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[mt], 0, 0, 0);
     }
     if constexpr (kc + 1 < MID_KC) StageReader<MT, kc + 1>::run(base, wbase, acc);
-  }
-  template <int mt>
-  static __device__ __forceinline__ void read_x(uint32_t base, u32x4 (&x)[MT]) {
-    x[mt] = lds_read16<(kc * SF + MID_WAVES + mt) * FRAG_BYTES>(base);
-    if constexpr (mt + 1 < MT) read_x<mt + 1>(base, x);
   }
 };
 
