@@ -105,7 +105,9 @@ __device__ __forceinline__ void store4(bf16* p, float4 v) {
   *reinterpret_cast<uint2*>(p) = u;
 }
 
-template <typename TX, typename TW, typename TY>
+// VEC: float4 groups a thread holds (the width is at most 4 * NORM_FAST_THREADS * VEC): as few as the width
+// needs, so that narrow rows do not pay in registers, and so in resident workgroups, for wide ones
+template <typename TX, typename TW, typename TY, int VEC>
 __global__ void __launch_bounds__(NORM_FAST_THREADS)
 add_rmsnorm_fast_kernel(const TX* __restrict__ x, float* __restrict__ stream, const TW* __restrict__ weight,
                         TY* __restrict__ y, const int* __restrict__ rows, int width, float eps) {
@@ -116,11 +118,11 @@ add_rmsnorm_fast_kernel(const TX* __restrict__ x, float* __restrict__ stream, co
   const TX* xr = x ? x + (size_t)row * width : nullptr;
   // first every load, as it comes from memory (a conversion or an add where a value is loaded would make
   // the compiler wait for it there, one memory latency per group of four instead of one in all)
-  Raw4<float> r_raw[NORM_FAST_VEC];
-  Raw4<TW> w_raw[NORM_FAST_VEC];
-  Raw4<TX> a_raw[NORM_FAST_VEC];
+  Raw4<float> r_raw[VEC];
+  Raw4<TW> w_raw[VEC];
+  Raw4<TX> a_raw[VEC];
 #pragma unroll
-  for (int k = 0; k < NORM_FAST_VEC; ++k) {
+  for (int k = 0; k < VEC; ++k) {
     const int i = (threadIdx.x + k * NORM_FAST_THREADS) * 4;
     r_raw[k] = Raw4<float>{};
     w_raw[k] = Raw4<TW>{};
@@ -131,9 +133,9 @@ add_rmsnorm_fast_kernel(const TX* __restrict__ x, float* __restrict__ stream, co
       if (xr) a_raw[k] = load_raw(xr + i);
     }
   }
-  float4 r[NORM_FAST_VEC], w[NORM_FAST_VEC];
+  float4 r[VEC], w[VEC];
 #pragma unroll
-  for (int k = 0; k < NORM_FAST_VEC; ++k) {
+  for (int k = 0; k < VEC; ++k) {
     r[k] = to_float4(r_raw[k]);
     w[k] = to_float4(w_raw[k]);
     const float4 a = to_float4(a_raw[k]);          // zeros where nothing was loaded
@@ -141,7 +143,7 @@ add_rmsnorm_fast_kernel(const TX* __restrict__ x, float* __restrict__ stream, co
   }
   float ss = 0.f;
 #pragma unroll
-  for (int k = 0; k < NORM_FAST_VEC; ++k) {
+  for (int k = 0; k < VEC; ++k) {
     ss = fmaf(r[k].x, r[k].x, ss); ss = fmaf(r[k].y, r[k].y, ss);
     ss = fmaf(r[k].z, r[k].z, ss); ss = fmaf(r[k].w, r[k].w, ss);
     const int i = (threadIdx.x + k * NORM_FAST_THREADS) * 4;
@@ -151,7 +153,7 @@ add_rmsnorm_fast_kernel(const TX* __restrict__ x, float* __restrict__ stream, co
   const float rstd = 1.0f / sqrtf(total / (float)width + eps);
   TY* yr = y + (size_t)out_row * width;
 #pragma unroll
-  for (int k = 0; k < NORM_FAST_VEC; ++k) {
+  for (int k = 0; k < VEC; ++k) {
     const int i = (threadIdx.x + k * NORM_FAST_THREADS) * 4;
     if (i < width)
       store4(yr + i, make_float4(r[k].x * rstd * w[k].x, r[k].y * rstd * w[k].y, r[k].z * rstd * w[k].z,
@@ -189,12 +191,22 @@ static int launch_norm(const void* x, float* stream, const void* w, void* y, int
   const bool fast = width % 4 == 0 && width <= 4 * NORM_FAST_THREADS * NORM_FAST_VEC &&
                     (((uintptr_t)x | (uintptr_t)stream | (uintptr_t)w | (uintptr_t)y) & 15) == 0;
   if (y_dtype != MIE_F32 && y_dtype != MIE_BF16) MIE_FAIL("add_rmsnorm: output dtype code %d", y_dtype);
-  if (fast && y_dtype == MIE_F32)
-    hipLaunchKernelGGL((add_rmsnorm_fast_kernel<TX, TW, float>), grid, dim3(NORM_FAST_THREADS), 0, s, (const TX*)x,
-                       stream, (const TW*)w, (float*)y, rows, width, eps);
-  else if (fast)
-    hipLaunchKernelGGL((add_rmsnorm_fast_kernel<TX, TW, bf16>), grid, dim3(NORM_FAST_THREADS), 0, s, (const TX*)x,
-                       stream, (const TW*)w, (bf16*)y, rows, width, eps);
+  if (fast) {
+#define NORM_FAST_LAUNCH(TY_, V_)                                                                                     \
+  hipLaunchKernelGGL((add_rmsnorm_fast_kernel<TX, TW, TY_, V_>), grid, dim3(NORM_FAST_THREADS), 0, s, (const TX*)x, \
+                     stream, (const TW*)w, (TY_*)y, rows, width, eps)
+    const int groups = (width / 4 + NORM_FAST_THREADS - 1) / NORM_FAST_THREADS;
+    if (y_dtype == MIE_F32) {
+      if (groups <= 2) NORM_FAST_LAUNCH(float, 2);
+      else if (groups <= 4) NORM_FAST_LAUNCH(float, 4);
+      else NORM_FAST_LAUNCH(float, NORM_FAST_VEC);
+    } else {
+      if (groups <= 2) NORM_FAST_LAUNCH(bf16, 2);
+      else if (groups <= 4) NORM_FAST_LAUNCH(bf16, 4);
+      else NORM_FAST_LAUNCH(bf16, NORM_FAST_VEC);
+    }
+#undef NORM_FAST_LAUNCH
+  }
   else if (y_dtype == MIE_F32)
     hipLaunchKernelGGL((add_rmsnorm_kernel<TX, TW, float>), grid, block, 0, s, (const TX*)x, stream, (const TW*)w,
                        (float*)y, rows, width, eps);

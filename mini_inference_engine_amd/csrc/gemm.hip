@@ -97,7 +97,11 @@ silu_mul_bf16x8_kernel(const bf16* __restrict__ gu, long ld_in, bf16* __restrict
     for (int j = 0; j < 4; ++j) {
       const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xFFFF0000u);
       const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xFFFF0000u);
-      const bf16 o0 = __float2bfloat16(g0 / (1.0f + expf(-g0)) * u0), o1 = __float2bfloat16(g1 / (1.0f + expf(-g1)) * u1);
+      // g / (1 + e^-g) by the hardware's exp2 and reciprocal (each within an ulp or two of the exact value, far
+      // below the bfloat16 rounding that follows): a tenth of the instructions of expf and a division
+      const float s0 = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g0 * -1.4426950408889634f));
+      const float s1 = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g1 * -1.4426950408889634f));
+      const bf16 o0 = __float2bfloat16(g0 * s0 * u0), o1 = __float2bfloat16(g1 * s1 * u1);
       ow[j] = (uint32_t)__builtin_bit_cast(uint16_t, o0) | ((uint32_t)__builtin_bit_cast(uint16_t, o1) << 16);
     }
     *reinterpret_cast<uint4*>(out + r * ld_out + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
