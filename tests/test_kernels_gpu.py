@@ -309,6 +309,36 @@ def test_many_row_projection_rotary_store(engine_ops, geom, slots_kind):
     assert torch.equal(vc.float().permute(0, 3, 1, 2)[keep], vc_ref.permute(0, 3, 1, 2)[keep]), "other slots' values stay"
 
 
+def test_projection_kernels_refuse_what_they_cannot_run(engine_ops):
+    """The entry points that take the projection's float32 sums name what is wrong instead of running."""
+    o = engine_ops
+    z = torch.zeros(64, device=DEV)
+    zi = torch.zeros(64, device=DEV, dtype=torch.int32)
+    zb = torch.zeros(4096, device=DEV, dtype=torch.bfloat16)
+    p = lambda t: t.data_ptr()
+    lib = o.lib("rope_kv")
+    # head size 20 is no multiple of 8; a page of 24 is no multiple of 16; leading dimension too short
+    assert lib.mie_rotary_kv_store_sums(p(z), 80, p(zb), 40, p(zi), p(z), p(z), p(zi), p(zb), p(zb), 2, 1, 20, 16, 1, None) != 0
+    assert b"multiple of 8" in lib._mie_error()
+    assert lib.mie_rotary_kv_store_sums(p(z), 64, p(zb), 32, p(zi), p(z), p(z), p(zi), p(zb), p(zb), 2, 1, 16, 24, 1, None) != 0
+    assert b"page" in lib._mie_error()
+    assert lib.mie_rotary_kv_store_sums(p(z), 48, p(zb), 32, p(zi), p(z), p(z), p(zi), p(zb), p(zb), 2, 1, 16, 16, 1, None) != 0
+    assert b"leading dims" in lib._mie_error()
+    assert lib.mie_rotary_kv_store_sums(None, 64, p(zb), 32, p(zi), p(z), p(z), p(zi), p(zb), p(zb), 2, 1, 16, 16, 1, None) != 0
+    assert b"null" in lib._mie_error()
+    lib = o.lib("attention_bf16", ("-DHEAD_DIM=16",))
+    args = lambda Hq, Hkv, D, splits, ld: (p(z), splits, 0, ld, p(z), p(z), p(zi), p(zb), p(zb), p(zb), p(zi), 4, p(zi), 1, Hq, Hkv, D,
+                                         16, 1.0, 0, lib.mie_decode_block_keys(), None)
+    assert lib.mie_decode_attention_from_sums(*args(34, 2, 16, 1, 608)) != 0
+    assert b"at most 16" in lib._mie_error()
+    assert lib.mie_decode_attention_from_sums(*args(4, 2, 32, 1, 256)) != 0
+    assert b"built for head_dim 16" in lib._mie_error()
+    assert lib.mie_decode_attention_from_sums(*args(4, 2, 16, 1, 100)) != 0
+    assert b"row stride" in lib._mie_error()
+    assert lib.mie_decode_attention_from_sums(*args(4, 2, 16, 3, 128)) != 0      # three splits with a stride of 0
+    assert b"splits" in lib._mie_error()
+
+
 def test_lazy_norm_input_adds_once(ops):
     """A Normed handed to linear: what is pending is added to the stream exactly once, however often it is used."""
     o = ops[torch.bfloat16]
