@@ -180,13 +180,19 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
       uint4 lo[PF_PPT], hi[PF_PPT];
     };
     int walk_idx = blk0 / page, walk_start = walk_idx * page;
+    // pages of a power of two (the usual 16): a key's page by a shift (the same for every lane)
+    const int page_shift = (page & (page - 1)) == 0 ? __builtin_ctz(page) : -1;
     auto lookup = [&](Where& Wh, int blk) {            // blocks are looked up in order, 64 keys apart
       blk = blk < last_blk ? blk : last_blk;           // beyond the last block: the last one again
       {
         const int d = blk - walk_start;
         int adv = 0;
+        if (page_shift >= 0) {
+          adv = d >> page_shift;
+        } else {
 #pragma unroll
-        for (int k = 1; k <= T16; ++k) adv += d >= k * page ? 1 : 0;
+          for (int k = 1; k <= T16; ++k) adv += d >= k * page ? 1 : 0;
+        }
         walk_start += adv * page;
         walk_idx += adv;
       }
@@ -203,8 +209,12 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
         }
         const int rel = key - walk_start;
         int w = 0;
+        if (page_shift >= 0) {
+          w = rel >> page_shift;
+        } else {
 #pragma unroll
-        for (int k = 1; k <= T16; ++k) w += rel >= k * page ? 1 : 0;
+          for (int k = 1; k <= T16; ++k) w += rel >= k * page ? 1 : 0;
+        }
         Wh.pg[i] = bt[walk_idx + w];
         Wh.off[i] = rel - w * page;
       }
