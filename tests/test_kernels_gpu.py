@@ -594,7 +594,7 @@ def test_decode_attention_split_count_and_static_bound(ops, ctx, splits):
 
 
 @pytest.mark.parametrize("geom", [(32, 4, 64, 16, 64), (8, 8, 128, 16, 40), (6, 2, 32, 32, 130), (16, 1, 16, 16, 257),
-                                  (10, 5, 48, 16, 52), (4, 4, 256, 16, 64)])
+                                  (10, 5, 48, 16, 52), (4, 4, 256, 16, 64), (16, 8, 64, 16, 64), (4, 4, 32, 16, 150)])
 @pytest.mark.parametrize("window", [None, 40])
 def test_decode_attention_finishes_the_projection(engine_ops, geom, window):
     """Steps of single-token rows whose rows x kv heads are 256 workgroups or more: the decode kernel takes the
@@ -602,7 +602,7 @@ def test_decode_attention_finishes_the_projection(engine_ops, geom, window):
     and does rotary, cache write and attention itself.  Against the same step done by the kernels that are each
     checked against their references elsewhere: sum + rotary + cache write, then attention over the cache.
     Contexts of 1 key, around the kernel's first blocks (which it asks for before the new key is written),
-    at page edges, and long ones."""
+    at page edges, and long ones; fewer and more than 512 workgroups (eight waves a workgroup, or four)."""
     from mini_inference_engine_amd.kernels.hip_backend import ProjectionSums
     from mini_inference_engine_amd.parts.rope import rotary_tables
     Hq, Hkv, D, page, M = geom
