@@ -465,16 +465,23 @@ class HipBackend(KernelBackend):
     DECODE_TARGET_WORKGROUPS = 512
     DECODE_WHOLE_WORKGROUPS = 256
 
-    def decode_splits(self, rows: int, Hq: int, Hkv: int, context_bound: int, window, block_keys: int):
+    def decode_splits(self, rows: int, Hq: int, Hkv: int, context_bound: int, window, block_keys: int,
+                      head_dim: int = 64):
         """(keys per split, number of splits) for single-token rows: split the context only as far
         as the rows and heads alone do not fill the GPU (inference_engine/kernels/decode_attention.py:117-125
-        follows the same idea), in whole blocks of the kernel."""
+        follows the same idea), in whole blocks of the kernel.
+
+        Not split at all (no partial results, no merge kernel): always when rows and heads give every compute unit
+        a workgroup; and with fewer workgroups where the contexts are short, because a workgroup then reads its
+        whole context in less time than the merge kernel takes.  Measured at head size 64 (keys of 256 bytes a kv
+        head): the unsplit kernel wins from 64 workgroups on at 512 keys, from 96 at 1,024, from 144 at 2,048:
+        about 32 + keys / 18."""
         if window:
             context_bound = min(context_bound, window + 32)
         base = rows * Hkv * -(-(Hq // Hkv) // 16)
         most = max(1, -(-context_bound // block_keys))
-        # rows and heads that give every compute unit a workgroup are not split: no partial results, no merge
-        target = self.DECODE_TARGET_WORKGROUPS if base < self.DECODE_WHOLE_WORKGROUPS else base
+        whole_from = min(self.DECODE_WHOLE_WORKGROUPS, 32 + context_bound * head_dim // (64 * 18))
+        target = self.DECODE_TARGET_WORKGROUPS if base < whole_from else base
         splits = max(1, min(-(-target // base), most))
         partition = -(-(-(-context_bound // splits)) // block_keys) * block_keys
         return partition, max(1, -(-context_bound // partition))
@@ -488,7 +495,7 @@ class HipBackend(KernelBackend):
             return None
         lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))
         block_keys = lib.mie_decode_block_keys()
-        partition, splits = self.decode_splits(T, Hq, Hkv, step.max_context, window, block_keys)
+        partition, splits = self.decode_splits(T, Hq, Hkv, step.max_context, window, block_keys, D)
         if splits != 1:
             return None
         part = pending.part
@@ -518,7 +525,7 @@ class HipBackend(KernelBackend):
             done = step.num_decode_rows        # single-token rows lead the batch: token t is row t
             lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))
             block_keys = lib.mie_decode_block_keys()
-            partition, splits = self.decode_splits(done, Hq, Hkv, step.max_context, window, block_keys)
+            partition, splits = self.decode_splits(done, Hq, Hkv, step.max_context, window, block_keys, D)
             if num_splits is not None:
                 bound = min(step.max_context, window + 32) if window else step.max_context
                 partition = -(-(-(-bound // num_splits)) // block_keys) * block_keys
