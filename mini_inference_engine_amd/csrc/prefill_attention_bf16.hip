@@ -29,10 +29,10 @@
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // Waves a workgroup, at head sizes up to 128 (above, eight waves do not fit the registers: always 4):
-// 8 over twice the queries where that still gives a workgroup to every compute unit (twice the queries share
-// each block that is brought in: at head size 128 and 8,192 tokens 0.82 against 0.40 PFLOP/s); for shorter
-// rows 8 in two halves over the keys, on the grid of 4: a wave's chain of blocks is half as long and every
-// SIMD has two waves (2,048 tokens at head size 64: 47 against 56 us).
+// 8 over twice the queries (twice the queries share each block that is brought in: at head size 128 and 8,192
+// tokens 0.82 against 0.40 PFLOP/s); for rows so short that the grid of 4 waves gives no more workgroups than
+// there are compute units, 8 in two halves over the keys on that grid: a wave's chain of blocks is half as
+// long and every SIMD has two waves (2,048 tokens at head size 64: 47 against 56 us).
 constexpr int PF_MAX_WAVES = D > 128 ? 4 : 8;
 constexpr bool PF_KEY_HALVES = D <= 128;            // (at 128 the two halves' kernel does not fit the registers)
 constexpr int PF_QW = 32;                           // queries a wave owns
@@ -472,10 +472,10 @@ MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k
   int waves_h;
   dim3 grid;
   if (PF_MAX_WAVES == 8) {
-    // (at head size 128 a compute unit holds one workgroup of the two-halves kind: more of them than compute
-    // units would run in two rounds, the second half empty)
-    const long n8 = plan(8, &waves_h, &grid), n4 = plan(4, &waves_h, &grid);
-    kind = n8 >= 256 || (D >= 128 && n4 > 256) ? EIGHT_QUERIES : EIGHT_KEYS;
+    // A compute unit holds one workgroup of eight waves (registers): more of the two-halves kind than compute
+    // units would run in two rounds, the second half empty (2,560 tokens: 95 us, against 45 for 2,048).
+    const long n4 = plan(4, &waves_h, &grid);
+    kind = n4 > 256 ? EIGHT_QUERIES : EIGHT_KEYS;
   }
   plan(kind == EIGHT_QUERIES ? 8 : 4, &waves_h, &grid);
   if (grid.y > 65535 || grid.z > 65535) MIE_FAIL("prefill_attention: grid too large (%d rows)", rows);
