@@ -32,9 +32,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // 8 over twice the queries (twice the queries share each block that is brought in: at head size 128 and 8,192
 // tokens 0.82 against 0.40 PFLOP/s); for rows so short that the grid of 4 waves gives no more workgroups than
 // there are compute units, 8 in two halves over the keys on that grid: a wave's chain of blocks is half as
-// long and every SIMD has two waves (2,048 tokens at head size 64: 47 against 56 us).
+// long and every SIMD has two waves (2,048 tokens at head size 64: 47 against 56 us).  Both kinds of eight
+// waves are built and used at every head size up to 128.
 constexpr int PF_MAX_WAVES = D > 128 ? 4 : 8;
-constexpr bool PF_KEY_HALVES = D <= 128;            // (at 128 the two halves' kernel does not fit the registers)
 constexpr int PF_QW = 32;                           // queries a wave owns
 constexpr int PF_BK = 64;                           // keys a step
 constexpr int KS16 = D / 16;                        // 16-dim steps of q . k
@@ -454,6 +454,13 @@ MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k
   const int G = Hq / Hkv;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) MIE_FAIL("prefill_attention: no current device");
+  static int compute_units[64] = {};              // of each device, asked for once
+  if (compute_units[dev] <= 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      MIE_FAIL("prefill_attention: cannot read the number of compute units of device %d", dev);
+    compute_units[dev] = n;
+  }
   // the grid for `waves` waves a workgroup: waves side by side over the heads of a group (a power of two), the rest
   // over 32-query tiles; a workgroup takes a late stretch and an early one
   auto plan = [&](int waves, int* waves_h, dim3* grid) {
@@ -475,7 +482,7 @@ MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k
     // A compute unit holds one workgroup of eight waves (registers): more of the two-halves kind than compute
     // units would run in two rounds, the second half empty (2,560 tokens: 95 us, against 45 for 2,048).
     const long n4 = plan(4, &waves_h, &grid);
-    kind = n4 > 256 ? EIGHT_QUERIES : EIGHT_KEYS;
+    kind = n4 > compute_units[dev] ? EIGHT_QUERIES : EIGHT_KEYS;
   }
   plan(kind == EIGHT_QUERIES ? 8 : 4, &waves_h, &grid);
   if (grid.y > 65535 || grid.z > 65535) MIE_FAIL("prefill_attention: grid too large (%d rows)", rows);

@@ -89,8 +89,9 @@ def normalise_config(cfg: dict) -> dict:
     return c
 
 
-def forward(cfg: dict, weights: dict, token_ids, dtype=torch.float64, position_offset: int = 0):
-    """Logits [n, vocab] of one whole sequence (inference_engine/model.py:161-185).
+def forward(cfg: dict, weights: dict, token_ids, dtype=torch.float64, position_offset: int = 0, rows=None):
+    """Logits [n, vocab] of one whole sequence (inference_engine/model.py:161-185); with ``rows`` (a list of
+    positions) only those rows of it, [len(rows), vocab], for sequences whose whole logits are too many.
     Residual wiring: stream = embed; stream += attention(norm(stream)); stream +=
     mlp(norm(stream)); logits = lm_head(norm(stream)).  ``position_offset`` shifts all
     positions (for the invariance test; the engine always starts at 0).  Runs where the
@@ -111,6 +112,8 @@ def forward(cfg: dict, weights: dict, token_ids, dtype=torch.float64, position_o
         x = rms_norm(stream, w[p + "post_attention_layernorm.weight"], eps)
         stream = stream + swiglu(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                                  w[p + "mlp.down_proj.weight"])
+    if rows is not None:
+        stream = stream[torch.as_tensor(rows, dtype=torch.long, device=device)]
     x = rms_norm(stream, w["model.norm.weight"], eps)
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
     return x @ head.T

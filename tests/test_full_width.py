@@ -208,3 +208,122 @@ def test_captured_step_of_160_rows_replayed(model):
         worst = max(worst, worst_error(got[i][None], expect[fed[i] - 1:fed[i]], BF16_TOL, f"request {i}",
                                        scale=float(expect.abs().max())))
     print(f"160-row captured step: four replays equal the eager step; worst {worst:.2e} of the logit scale")
+
+
+# ------------------------------------------------------------------ the cuts of the replay tests, at these widths
+LONG = [640, 700, 610, 820, 660, 600]
+
+
+def compare_trace(model, dtype, prompts, got, what):
+    tol = F32_TOL if dtype == "float32" else BF16_TOL
+    assert len(got) == sum(len(t) for t in prompts.values())
+    worst = 0.0
+    for rid, toks in prompts.items():
+        expect = plain_logits(model, dtype, toks)
+        rows = torch.stack([got[(rid, p)] for p in range(len(toks))])
+        worst = max(worst, worst_error(rows, expect, tol, f"{what}: request {rid}"))
+    return worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_portions_of_changing_size_at_full_width(model, dtype):
+    """Two prompts of 640 and 700 tokens in portions from 2 to 257 tokens: later portions read several 64-key
+    blocks of earlier ones through the block table, start and end inside pages, and the portions of more than
+    128 tokens take the many-row products (library product, rotary and cache write from its float32 sums) while
+    the short ones take the few-row kernels; every position's logits against the plain implementation."""
+    import trace_util
+    prompts = {k: v for k, v in list(trace_util.random_prompts(CFG["vocab_size"], LONG, seed=41).items())[:2]}
+    steps = trace_util.portions(prompts, sizes=(200, 2, 150, 7, 129, 3, 64, 33, 257, 2, 16, 70))
+    assert min(len(e["tokens"]) for s in steps for e in s["entries"]) == 2
+    assert max(len(e["tokens"]) for s in steps for e in s["entries"]) > 128
+    peak = trace_util.live_token_peak(steps)
+    runner = make_runner(model, dtype, pages=peak // 16 + 1, max_rows=4, max_step_tokens=512)
+    got = trace_util.run_on_runner(runner, steps)
+    runner.cache.check()
+    worst = compare_trace(model, dtype, prompts, got, f"{dtype}: portions")
+    print(f"{dtype}: portions of 2 to 257 tokens at full width, worst {worst:.2e} of the logit scale")
+
+
+@pytest.mark.parametrize("captured", [False, True], ids=["eager", "graphs"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_steps_with_pages_used_again_at_full_width(model, dtype, captured):
+    """Six requests of 600 to 820 tokens, four live at a time, portions of 2 to 257 tokens of some beside single
+    tokens of others (steps of up to several hundred tokens), in a pool smaller than all requests together, so
+    that later requests run in pages earlier ones gave back."""
+    import trace_util
+    prompts = trace_util.random_prompts(CFG["vocab_size"], LONG, seed=43)
+    steps = trace_util.mixed(prompts, max_live=4, seed=3, tail=10, sizes=(2, 3, 17, 64, 130, 200, 257))
+    assert max(sum(len(e["tokens"]) for e in s["entries"]) for s in steps) > 256
+    assert any(len(e["tokens"]) == 1 for s in steps for e in s["entries"] if len(s["entries"]) > 1
+               and max(len(f["tokens"]) for f in s["entries"]) > 128)
+    peak = trace_util.live_token_peak(steps)
+    assert peak // 16 < sum(-(-n // 16) for n in LONG), "the pool must be smaller than all requests together"
+    runner = make_runner(model, dtype, pages=peak // 16 + 1, max_rows=8, max_step_tokens=1024)
+    if captured:
+        runner.capture_decode_graphs((1, 2, 4))
+    got = trace_util.run_on_runner(runner, steps)
+    runner.cache.check()
+    worst = compare_trace(model, dtype, prompts, got, f"{dtype}: mixed")
+    print(f"{dtype}: mixed steps at full width ({len(steps)} steps, pool {peak // 16 + 1} pages), "
+          f"worst {worst:.2e} of the logit scale")
+
+
+SWEEP = (24, 33, 65, 96, 128, 129, 256)
+
+
+@pytest.mark.parametrize("captured", [False, True], ids=["eager", "graphs"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_from_24_to_256_rows(model, dtype, captured):
+    """One step of single-token rows at each of 24, 33, 65, 96, 128, 129 and 256 rows, launched kernel by kernel
+    and through captured graphs of exactly those sizes: the row counts at which the products change kernel
+    (few-row kernel to 32 rows, split product to 64, or to 128 for the down projection, the library beyond) and
+    at which the decode attention stops splitting contexts.  A sample of each step's rows against the plain
+    implementation."""
+    from mini_inference_engine_amd.engine.batch import StepRow
+    tol = F32_TOL if dtype == "float32" else BF16_TOL
+    n_req, ahead = max(SWEEP), len(SWEEP)
+    lengths = [10 + (i * 37) % 64 for i in range(n_req)]
+    requests = [prompt_tokens(n, 2000 + i) for i, n in enumerate(lengths)]
+    runner = make_runner(model, dtype, pages=sum(-(-n // 16) for n in lengths) + 1, max_rows=n_req, max_step_tokens=2048)
+    if captured:
+        runner.capture_decode_graphs(SWEEP)
+    caches = [runner.cache.open(i) for i in range(n_req)]
+    fed = [0] * n_req
+
+    def feed(which, counts, want_last):
+        rows = []
+        for i, n in zip(which, counts):
+            assert runner.cache.reserve(caches[i], fed[i], n)
+            rows.append(StepRow(caches[i], requests[i][fed[i]:fed[i] + n], fed[i], [n - 1] if want_last else []))
+        out = runner.forward_step(rows)
+        for i, n in zip(which, counts):
+            fed[i] += n
+        return out
+
+    batch, room = [], 2048
+    for i, n in enumerate(lengths):                      # all but the last ``ahead`` tokens as prompts
+        if n - ahead > room:
+            feed(batch, [lengths[j] - ahead for j in batch], False)
+            batch, room = [], 2048
+        batch.append(i)
+        room -= n - ahead
+    feed(batch, [lengths[j] - ahead for j in batch], False)
+
+    got = {}
+    for n in SWEEP:
+        out = feed(range(n), [1] * n, True)
+        assert runner.last_step_captured == captured
+        for i in sorted({0, 1, n // 2, n - 2, n - 1} | set(range(7, n, 40))):
+            got[(n, i, fed[i] - 1)] = out[i].clone()
+    worst, expect_of = 0.0, {}
+    for (n, i, p), row in got.items():
+        if i not in expect_of:
+            expect_of[i] = plain_logits(model, dtype, requests[i])
+        e = expect_of[i]
+        worst = max(worst, worst_error(row[None], e[p:p + 1], tol, f"{dtype}/{'graphs' if captured else 'eager'}: "
+                                       f"step of {n} rows, row {i}, position {p}", scale=float(e.abs().max())))
+    for rc in caches:
+        runner.cache.close(rc)
+    runner.cache.check()
+    print(f"{dtype}/{'graphs' if captured else 'eager'}: steps of {SWEEP} rows, {len(got)} rows checked, "
+          f"worst {worst:.2e} of the logit scale")

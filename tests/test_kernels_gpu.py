@@ -457,7 +457,8 @@ def test_rotary_kv_store(ops, dtype, geom):
     assert torch.equal(kc[0], kc_ref[0]) and torch.equal(vc[0], vc_ref[0])
 
 
-@pytest.mark.parametrize("geom", [(2, 1, 16), (3, 1, 32), (4, 2, 48), (32, 4, 64), (3, 3, 80), (5, 5, 96), (8, 2, 128), (2, 1, 256)])
+@pytest.mark.parametrize("geom", [(2, 1, 16), (3, 1, 32), (4, 2, 48), (32, 4, 64), (3, 3, 80), (5, 5, 96), (8, 2, 128), (2, 1, 256),
+                                  (3, 1, 112), (2, 2, 192)])
 @pytest.mark.parametrize("M", [1, 8, 16, 40])
 def test_fused_projection_rotary_store(ops, geom, M):
     """Projection + rotary + cache write in one kernel against the three separate references."""
@@ -593,8 +594,83 @@ def test_decode_attention_split_count_and_static_bound(ops, ctx, splits):
     torch.testing.assert_close(out2.double(), expect, **ATT_TOL[dtype])
 
 
+LONG_DECODE = [  # (Hq, Hkv, D), contexts
+    ((32, 4, 64), [4096]), ((32, 4, 64), [8192]), ((32, 8, 128), [8192]), ((32, 32, 128), [4096]),
+    ((32, 8, 128), [8191, 5, 4097, 300, 6000, 64, 1, 2048]),
+    ((32, 8, 128), [8192] + [40 + 3 * i for i in range(63)]),        # 64 rows: rows x kv heads fill the GPU, no split
+]
+
+
+@pytest.mark.parametrize("spiked", [False, True], ids=["random", "far key"])
+@pytest.mark.parametrize("splits", [None, 1, 64])
+@pytest.mark.parametrize("case", LONG_DECODE, ids=[f"{g[0]}on{g[1]}x{g[2]}-{len(c)}rows-{max(c)}" for g, c in LONG_DECODE])
+def test_decode_attention_past_4096_keys(ops, case, splits, spiked):
+    """Contexts of 4,096 and 8,192 keys (block tables of 256 and 512 pages) at the head sizes and groupings of the
+    benchmark configurations: with the split the engine chooses (up to 64 partial results a head for one row,
+    none for 64 rows), unsplit, and split 64 ways; with random keys, and with one key among the first 64 made to
+    dominate the longest row's query, 8,000 keys away."""
+    (Hq, Hkv, D), ctx = case
+    dtype = torch.bfloat16
+    spike = (0, 37) if spiked else None
+    q, kc, vc, group, step = paged_setup(ctx, [1] * len(ctx), Hq, Hkv, D, 16, dtype, seed=len(ctx) + D, spike=spike)
+    scale = 1.0 if spiked else 1 / math.sqrt(D)
+    out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, scale, None, num_splits=splits)
+    torch.testing.assert_close(out.double(), expect, **(SPIKE_TOL if spiked else ATT_TOL)[dtype])
+    if spiked:          # the far key's value is what comes out
+        pg = int(group.block_tables[0, 37 // 16])
+        v_far = vc[pg, :, :, 37 % 16].float().repeat_interleave(Hq // Hkv, dim=0).reshape(-1)
+        torch.testing.assert_close(out[0].float(), v_far, atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("key", [None, 5, 6143, 6144, 8100])
+@pytest.mark.parametrize("geom", [(32, 8, 128), (32, 4, 64)])
+def test_prefill_attention_with_6144_earlier_tokens(ops, geom, key):
+    """A portion of 2,048 tokens behind 6,144 earlier ones (and a short portion behind 6,144 beside it): the walk
+    over a block table of 512 pages, 128 blocks of 64 keys a query tile.  A sample of the queries against the
+    token-by-token reference; with ``key``, that key is made to dominate the last query."""
+    Hq, Hkv, D = geom
+    dtype = torch.bfloat16
+    ctx, qn = [8192, 6200], [2048, 56]
+    q, kc, vc, group, step = paged_setup(ctx, qn, Hq, Hkv, D, 16, dtype, seed=D + (key or 0),
+                                         spike=None if key is None else (0, key))
+    scale = 1 / math.sqrt(D) if key is None else 1.0
+    out = ops[dtype].paged_attention(q, Hq, Hkv, D, kc, vc, group, step, scale, None)
+    idx = torch.tensor([0, 1, 15, 16, 31, 32, 63, 64, 65, 1000, 1023, 1024, 2046, 2047, 2048, 2049, 2103], device=DEV)
+    expect = ref.ref_paged_attention(q[idx], Hq, Hkv, D, kc, vc, group.block_tables, step.token_row[idx],
+                                     step.positions[idx], scale, None, torch.float64)
+    torch.testing.assert_close(out[idx].double(), expect, **(ATT_TOL if key is None else SPIKE_TOL)[dtype])
+    assert bool(torch.isfinite(out.float()).all())
+
+
+@pytest.mark.parametrize("D", [112, 192])
+def test_head_sizes_outside_the_prebuilt_list(ops, D):
+    """Head sizes that are a multiple of 16 but not in kernels/variants.py: the attention modules for them are
+    compiled at first use (unless an earlier run left them built) and must give what the others give: decode
+    attention split and unsplit, prefill attention behind earlier portions and with a window, a far key, against
+    the references.  (The projection kernels take the head size at run time: 112 and 192 are among the geometries
+    of test_fused_projection_rotary_store and test_decode_attention_finishes_the_projection.)"""
+    from mini_inference_engine_amd.kernels.variants import HEAD_DIMS
+    assert D not in HEAD_DIMS and D % 16 == 0
+    dtype = torch.bfloat16
+    Hq, Hkv, page = 6, 2, 16
+    for splits in (None, 1, 5):
+        q, kc, vc, group, step = paged_setup([1, 17, 700, 64, 65, 1500], [1] * 6, Hq, Hkv, D, page, dtype, seed=D)
+        out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1 / math.sqrt(D), None,
+                                    num_splits=splits)
+        torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+    for window in (None, 24):
+        q, kc, vc, group, step = paged_setup([9, 300, 2, 64, 65, 200, 1000], [1, 1, 2, 64, 65, 3, 489], Hq, Hkv, D, page,
+                                             dtype, seed=D + 1)
+        out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1.1 / math.sqrt(D), window)
+        torch.testing.assert_close(out.double(), expect, **ATT_TOL[dtype])
+    q, kc, vc, group, step = paged_setup([600], [600], Hq, Hkv, D, page, dtype, seed=D + 2, spike=(0, 3))
+    out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, 1.0, None)
+    torch.testing.assert_close(out.double(), expect, **SPIKE_TOL[dtype])
+
+
 @pytest.mark.parametrize("geom", [(32, 4, 64, 16, 64), (8, 8, 128, 16, 40), (6, 2, 32, 32, 130), (16, 1, 16, 16, 257),
-                                  (10, 5, 48, 16, 52), (4, 4, 256, 16, 64), (16, 8, 64, 16, 64), (4, 4, 32, 16, 150)])
+                                  (10, 5, 48, 16, 52), (4, 4, 256, 16, 64), (16, 8, 64, 16, 64), (4, 4, 32, 16, 150),
+                                  (4, 2, 112, 16, 130), (4, 4, 192, 16, 64)])
 @pytest.mark.parametrize("window", [None, 40])
 def test_decode_attention_finishes_the_projection(engine_ops, geom, window):
     """Steps of single-token rows whose rows x kv heads are 256 workgroups or more: the decode kernel takes the

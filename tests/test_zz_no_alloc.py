@@ -56,12 +56,18 @@ def _both(lib, ctx, splits, seed):
                                   c_void_p(out_a.data_ptr()), c_void_p(o_part.data_ptr()),
                                   c_void_p(lse_part.data_ptr()), *shared)
     assert rc == 0, lib.attention_bf16_last_error()
+    torch.cuda.synchronize()
+    # what the driver itself says is free on the device: a hipMalloc inside the library would show here (torch's
+    # own counters see only torch's allocator); the kernels' code was loaded by the call above
+    free_before, _ = torch.cuda.mem_get_info()
     before = torch.cuda.memory_allocated()
     rc = lib.mie_decode_attention_static(c_void_p(q.data_ptr()), q.stride(0), c_void_p(kc.data_ptr()),
                                          c_void_p(vc.data_ptr()), c_void_p(out_b.data_ptr()), *shared)
     assert rc == 0, lib.attention_bf16_last_error()
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, f"device memory free before the call {free_before}, after it {free_after}"
     expect = ref.ref_paged_attention(q, Hq, Hkv, D, kc, vc, bt, step.token_row, step.positions, scale, None,
                                      torch.float64)
     return out_a, out_b, expect, n
@@ -77,6 +83,56 @@ def test_static_decode_attention_equals_the_one_with_buffers():
         assert n == splits
         assert torch.equal(out_a, out_b), f"contexts {ctx}, {n} splits: the two entry points differ"
         torch.testing.assert_close(out_b.double(), expect, atol=2e-2, rtol=2e-2)
+
+
+def test_static_decode_attention_inside_a_captured_graph():
+    """The use the entry point is for: set-up once, then the call recorded into a graph (where an allocation is
+    an error that ends the capture) and replayed with other inputs in the same buffers, with eager work and
+    synchronisations between the replays; every replay against the entry point that takes buffers."""
+    lib = _library()
+    assert lib.mie_decode_attention_static_setup() == 0, lib.attention_bf16_last_error()
+    ctx, splits = [5, 300, 1, 2047, 64, 65], 8
+    rows = len(ctx)
+    q, kc, vc, group, step = paged_setup(ctx, [1] * rows, Hq, Hkv, D, PAGE, torch.bfloat16, seed=21)
+    bt = group.block_tables
+    partition, n = _split(lib, max(ctx), splits)
+    scale = 1 / math.sqrt(D)
+    out_g = torch.zeros(rows, Hq * D, dtype=torch.bfloat16, device="cuda")
+    o_part = torch.empty(rows, Hq, n, D, dtype=torch.float32, device="cuda")
+    lse_part = torch.empty(rows, Hq, n, dtype=torch.float32, device="cuda")
+
+    def shared(stream):
+        return [c_void_p(bt.data_ptr()), bt.shape[1], c_void_p(step.positions.data_ptr()), rows, Hq, Hkv, D, PAGE,
+                scale, 0, partition, n, c_void_p(stream)]
+
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.mie_decode_attention_static(c_void_p(q.data_ptr()), q.stride(0), c_void_p(kc.data_ptr()),
+                                             c_void_p(vc.data_ptr()), c_void_p(out_g.data_ptr()),
+                                             *shared(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, lib.attention_bf16_last_error()
+    for replay in range(3):
+        if replay:                  # other queries and other keys in the same buffers
+            g = torch.Generator(device="cuda").manual_seed(100 + replay)
+            q.copy_(torch.randn(q.shape, generator=g, device="cuda"))
+            kc.copy_(torch.randn(kc.shape, generator=g, device="cuda"))
+        out_g.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        out_a = torch.zeros_like(out_g)
+        rc = lib.mie_decode_attention(c_void_p(q.data_ptr()), q.stride(0), c_void_p(kc.data_ptr()),
+                                      c_void_p(vc.data_ptr()), c_void_p(out_a.data_ptr()), c_void_p(o_part.data_ptr()),
+                                      c_void_p(lse_part.data_ptr()), *shared(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, lib.attention_bf16_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_a), f"replay {replay} of the recorded call differs from the call with buffers"
+        expect = ref.ref_paged_attention(q, Hq, Hkv, D, kc, vc, bt, step.token_row, step.positions, scale, None,
+                                         torch.float64)
+        torch.testing.assert_close(out_g.double(), expect, atol=2e-2, rtol=2e-2)
+    del graph
+    torch.cuda.synchronize()
 
 
 def test_static_decode_attention_refuses_what_does_not_fit():

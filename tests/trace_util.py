@@ -59,9 +59,10 @@ def portions(prompts: dict, sizes=(7, 2, 16, 3, 2, 33, 5, 2, 64)) -> list:
     return steps
 
 
-def mixed(prompts: dict, max_live: int = 4, seed: int = 0, tail: int = 12) -> list:
-    """Requests enter as slots free up; each is fed in portions of random size, then its
-    last ``tail`` tokens one at a time, so steps mix portions with single tokens; some
+def mixed(prompts: dict, max_live: int = 4, seed: int = 0, tail: int = 12,
+          sizes=(2, 3, 5, 8, 13, 16, 17, 31)) -> list:
+    """Requests enter as slots free up; each is fed in portions of random size (one of ``sizes``), then
+    its last ``tail`` tokens one at a time, so steps mix portions with single tokens; some
     requests sit a step out now and then."""
     rng = np.random.default_rng(seed)
     waiting = list(prompts.items())
@@ -80,7 +81,7 @@ def mixed(prompts: dict, max_live: int = 4, seed: int = 0, tail: int = 12) -> li
             if left <= tail:
                 m = 1
             else:
-                m = int(min(left - tail, rng.choice([2, 3, 5, 8, 13, 16, 17, 31])))
+                m = int(min(left - tail, rng.choice(list(sizes))))
                 if m == 1:
                     m = min(2, left)
             entries.append({"id": rid, "tokens": toks[p:p + m], "want": list(range(m))})
@@ -104,6 +105,36 @@ def live_token_peak(steps: list, round_to: int = 64) -> int:
         for rid in s["end"]:
             held.pop(rid, None)
     return peak
+
+
+def run_on_runner(runner, steps: list) -> dict:
+    """Runs a trace's steps on a ModelRunner as replay does (open, reserve, forward_step, after_step, close) but
+    keeps what it computes where it is: (request id, position) -> logits row on the runner's device.  For models
+    whose logits are too many to go through files."""
+    from mini_inference_engine_amd.engine.batch import StepRow
+    live, got = {}, {}
+    for s in steps:
+        rows = []
+        for e in s["entries"]:
+            if e["id"] not in live:
+                live[e["id"]] = [runner.cache.open(e["id"]), 0]
+            rc, have = live[e["id"]]
+            assert runner.cache.reserve(rc, have, len(e["tokens"])), f"step {s['step']}: out of pages"
+            rows.append(StepRow(rc, e["tokens"], have, list(e.get("want", []))))
+        logits = runner.forward_step(rows)
+        runner.after_step(rows)
+        k = 0
+        for e in s["entries"]:
+            base = live[e["id"]][1]
+            for w in e.get("want", []):
+                got[(e["id"], base + w)] = logits[k].clone()      # a captured step's logits are overwritten by the next
+                k += 1
+            live[e["id"]][1] = base + len(e["tokens"])
+        assert k == (0 if logits is None else logits.shape[0])
+        for rid in s["end"]:
+            runner.cache.close(live.pop(rid)[0])
+    assert not live, "the trace left requests open"
+    return got
 
 
 def to_lines(steps: list) -> list:
