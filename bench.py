@@ -44,14 +44,11 @@ SHAPE_NAMES = {"tinyllama": "TinyLlama-1.1B", "llama2-7b": "Llama-2-7B", "llama3
 
 
 def shape_config(shape: str = "tinyllama", layers: int | None = None):
-    """Layer sizes by name (the command line's table); ``layers``: fewer layers than the model has."""
-    from mini_inference_engine_amd.__main__ import SHAPES
-    from mini_inference_engine_amd.config import LlamaConfig
-    d = dict(SHAPES[shape], architectures=["LlamaForCausalLM"], eos_token_id=2)
-    full = d["num_hidden_layers"]
-    if layers:
-        d["num_hidden_layers"] = layers
-    return LlamaConfig.from_dict(d), full
+    """Layer sizes by name (the named sizes the architecture registered); ``layers``: fewer layers than the
+    model has.  Returns the configuration and the number of layers the named size has."""
+    from mini_inference_engine_amd.config import registry
+    full = registry.shape_config(shape).num_hidden_layers
+    return registry.shape_config(shape, **({"num_hidden_layers": layers} if layers else {})), full
 
 
 def tinyllama_config(layers: int | None = None):
@@ -252,7 +249,7 @@ def measure_kernels(cfg, args) -> int:
     step = SimpleNamespace(token_row=torch.arange(M, device=dev, dtype=torch.int32), positions=pos, num_rows=M,
                            max_context=ctx, num_tokens=M, num_decode_rows=M, max_row_tokens=1, row_start=None,
                            row_position=None)
-    group = SimpleNamespace(block_tables=bt, max_blocks=bt.shape[1])
+    group = SimpleNamespace(block_tables=bt, max_blocks=bt.shape[1], slot_mapping=slots)
     t = timed(lambda i: ops.paged_attention(qkv, Hq, Hkv, D, kc, vc, group, step, D ** -0.5, None), 8)
     report(f"decode attention + merge, {M} rows of {ctx} keys", t, 2 * 2 * M * ctx * Hkv * D)
     # ---- the q/k/v projection and the attention as the engine runs them in a step of M single-token rows

@@ -14,29 +14,14 @@ import json
 import sys
 import tempfile
 
-SHAPES = {
-    # the two tiny configurations of the tests, the benchmark's layer sizes, and two larger models' sizes
-    "tiny-a": dict(vocab_size=256, hidden_size=64, intermediate_size=176, num_hidden_layers=2, num_attention_heads=4,
-                   num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-5, rope_theta=10000.0,
-                   max_position_embeddings=128, tie_word_embeddings=False),
-    "tiny-b": dict(vocab_size=384, hidden_size=96, intermediate_size=256, num_hidden_layers=3, num_attention_heads=3,
-                   num_key_value_heads=1, head_dim=32, rms_norm_eps=1e-6, rope_theta=500000.0,
-                   max_position_embeddings=256, tie_word_embeddings=True),
-    "tinyllama": dict(vocab_size=32000, hidden_size=2048, intermediate_size=5632, num_hidden_layers=22,
-                      num_attention_heads=32, num_key_value_heads=4, head_dim=64, rms_norm_eps=1e-5,
-                      rope_theta=10000.0, max_position_embeddings=2048, tie_word_embeddings=False),
-    "llama2-7b": dict(vocab_size=32000, hidden_size=4096, intermediate_size=11008, num_hidden_layers=32,
-                      num_attention_heads=32, num_key_value_heads=32, head_dim=128, rms_norm_eps=1e-5,
-                      rope_theta=10000.0, max_position_embeddings=4096, tie_word_embeddings=False),
-    "llama3-8b": dict(vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_hidden_layers=32,
-                      num_attention_heads=32, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-5,
-                      rope_theta=500000.0, max_position_embeddings=8192, tie_word_embeddings=False),
-}
-
-
 def _shape_config(name: str):
-    from .config import LlamaConfig
-    return LlamaConfig.from_dict({**SHAPES[name], "architectures": ["LlamaForCausalLM"]})
+    from .config.registry import shape_config
+    return shape_config(name)
+
+
+def _shapes() -> list[str]:
+    from .config.registry import known_shapes
+    return known_shapes()
 
 
 def _ints(text: str) -> list[int]:
@@ -45,7 +30,8 @@ def _ints(text: str) -> list[int]:
 
 def _add_model_args(ap):
     ap.add_argument("--model", help="folder with config.json and safetensors")
-    ap.add_argument("--shape", choices=sorted(SHAPES), help="random weights at a named size instead of --model")
+    ap.add_argument("--shape", choices=_shapes(),
+                    help="random weights at a named size of a registered architecture instead of --model")
     ap.add_argument("--seed", type=int, default=0, help="seed of the random weights and of sampling")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "bf16", "float32", "fp32"])
 
@@ -136,7 +122,7 @@ def main(argv=None) -> int:
     g.set_defaults(fn=cmd_generate)
 
     r = sub.add_parser("random-model", help="write config.json and model.safetensors with random weights")
-    r.add_argument("--shape", choices=sorted(SHAPES))
+    r.add_argument("--shape", choices=_shapes())
     r.add_argument("--config", help="a config.json (or its folder) instead of --shape")
     r.add_argument("--seed", type=int, default=0)
     r.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "bf16", "float32", "fp32"])

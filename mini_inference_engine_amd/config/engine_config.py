@@ -5,7 +5,8 @@ Names and meanings follow the reference's EngineConfig
 max_num_batched_tokens, kv_cache_memory_fraction, max_model_len,
 enable_chunked_prefill.  Its Triton and CUDA-graph switches become one
 ``use_hip_graphs`` switch with ``graph_batch_sizes``; ``num_blocks`` (an explicit
-page count), ``num_state_slots`` and ``seed`` have no counterpart there.
+page count), ``num_state_slots``, ``seed`` and ``cast_float32_weights`` have no
+counterpart there.
 """
 from __future__ import annotations
 
@@ -28,6 +29,8 @@ class EngineConfig:
     activation_reserve_bytes: int = 768 * 2**20
     poison_freed_pages: bool = False        # debugging: fill returned pages with NaN
     run_ahead: bool = True                  # start a step before the host has read the tokens of the one before
+    cast_float32_weights: bool = False      # bfloat16 mode: round tensors the checkpoint stores in 32-bit to bfloat16
+                                            # (the reference casts every tensor; by default they stay as stored)
 
     def __post_init__(self):
         if self.block_size < 16 or self.block_size % 16:

@@ -72,7 +72,8 @@ class LlamaConfig(ModelConfig):
     required are vocab_size, hidden_size, intermediate_size, num_hidden_layers,
     num_attention_heads, rms_norm_eps, max_position_embeddings; num_key_value_heads
     defaults to the head count, head_dim to hidden_size // heads, rope_theta to
-    10000, tie_word_embeddings to false, eos_token_id to 2 (first entry of a list).
+    10000, tie_word_embeddings to false, eos_token_id to 2.  The reference keeps the first entry of a list of
+    stop ids; here every entry stops a request (``eos_token_id`` is the tuple of them).
     """
 
     vocab_size: int
@@ -86,7 +87,7 @@ class LlamaConfig(ModelConfig):
     rope_theta: float
     max_position_embeddings: int
     tie_word_embeddings: bool = False
-    eos_token_id: int = 2
+    eos_token_id: tuple = (2,)
 
     architecture = "LlamaForCausalLM"
 
@@ -118,10 +119,11 @@ class LlamaConfig(ModelConfig):
                 raise ConfigError(f"config.json: {key}=true is not computed here")
         head_dim = d.get("head_dim") or hidden // heads
         eos = d.get("eos_token_id", 2)
-        if isinstance(eos, list):
-            if not eos:
-                raise ConfigError("config.json: eos_token_id is an empty list")
-            eos = eos[0]
+        if not isinstance(eos, (list, tuple)):
+            eos = [eos]
+        if not eos:
+            raise ConfigError("config.json: eos_token_id is an empty list")
+        eos = tuple(_take_int({"eos_token_id": e}, "eos_token_id", minimum=0) for e in eos)
         return cls(
             vocab_size=_take_int(d, "vocab_size"),
             hidden_size=hidden,
@@ -134,11 +136,12 @@ class LlamaConfig(ModelConfig):
             rope_theta=_take_float(d, "rope_theta", default=10000.0),
             max_position_embeddings=_take_int(d, "max_position_embeddings"),
             tie_word_embeddings=_take_bool(d, "tie_word_embeddings", False),
-            eos_token_id=_take_int({"eos_token_id": eos}, "eos_token_id", minimum=0),
+            eos_token_id=eos,
         )
 
     def to_dict(self) -> dict:
         d = asdict(self)
+        d["eos_token_id"] = self.eos_token_id[0] if len(self.eos_token_id) == 1 else list(self.eos_token_id)
         d["architectures"] = [self.architecture]
         d["model_type"] = "llama"
         d["hidden_act"] = "silu"

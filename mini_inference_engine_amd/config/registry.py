@@ -20,6 +20,7 @@ class Architecture:
     name: str
     config_type: type
     build: Callable[[Any], Any]
+    shapes: Mapping[str, Mapping[str, Any]] = None     # named sizes: shape name -> config.json keys
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}
@@ -27,10 +28,16 @@ _MODEL_TYPES: dict[str, str] = {}
 
 
 def register_architecture(name: str, config_type: type, build: Callable, *, model_type: str | None = None,
-                          replace: bool = False) -> None:
+                          shapes: Mapping[str, Mapping[str, Any]] | None = None, replace: bool = False) -> None:
+    """``shapes``: sizes of this architecture that have a name (``--shape`` of the command line and of the
+    benchmark): shape name -> the config.json keys of that size, without ``architectures``."""
     if name in _ARCHITECTURES and not replace:
         raise ValueError(f"architecture '{name}' is already registered")
-    _ARCHITECTURES[name] = Architecture(name, config_type, build)
+    for shape in shapes or {}:
+        owner = next((a.name for a in _ARCHITECTURES.values() if a.name != name and shape in (a.shapes or {})), None)
+        if owner:
+            raise ValueError(f"shape '{shape}' is already a named size of architecture '{owner}'")
+    _ARCHITECTURES[name] = Architecture(name, config_type, build, dict(shapes or {}))
     if model_type is not None:
         _MODEL_TYPES[model_type] = name
 
@@ -39,6 +46,22 @@ def unregister_architecture(name: str) -> None:
     _ARCHITECTURES.pop(name, None)
     for k in [k for k, v in _MODEL_TYPES.items() if v == name]:
         del _MODEL_TYPES[k]
+
+
+def known_shapes() -> list[str]:
+    """Every named size of every registered architecture."""
+    _ensure_builtin()
+    return sorted(shape for a in _ARCHITECTURES.values() for shape in (a.shapes or {}))
+
+
+def shape_config(shape: str, **overrides) -> ModelConfig:
+    """The typed configuration of a named size; ``overrides`` replace config.json keys of it (fewer layers,
+    say) before it is read."""
+    _ensure_builtin()
+    for a in _ARCHITECTURES.values():
+        if shape in (a.shapes or {}):
+            return a.config_type.from_dict({**a.shapes[shape], **overrides, "architectures": [a.name]})
+    raise ConfigError(f"no registered architecture has a size named '{shape}'; known: {known_shapes()}")
 
 
 def known_architectures() -> list[str]:

@@ -54,7 +54,7 @@ class LLMEngine:
             num_pages=cfg.num_blocks, memory_fraction=cfg.kv_cache_memory_fraction,
             reserve_bytes=cfg.activation_reserve_bytes, max_step_tokens=cfg.max_num_batched_tokens,
             max_rows=cfg.max_num_seqs, max_model_len=cfg.max_model_len, num_state_slots=cfg.num_state_slots,
-            weights=weights)
+            weights=weights, cast_float32_weights=cfg.cast_float32_weights)
         self.model_cfg = self.runner.model_cfg
         self.cfg.max_model_len = self.runner.max_model_len
         self.cache = self.runner.cache
@@ -64,7 +64,7 @@ class LLMEngine:
         self.scheduler = Scheduler(self.cfg, self.cache)
         self.sampler = Sampler(self.runner.ops, self.runner.device, cfg.max_num_seqs, out=self.runner.chosen_tokens)
         self._in_flight = None             # the step whose tokens the host has not read yet
-        self.eos_token_id = self.runner.model.spec.eos_token_id
+        self.stop_token_ids = frozenset(self.runner.model.spec.stop_token_ids)
         if verbose:
             print(f"[mini_inference_engine_amd] cache: {self.runner.num_pages} pages x {cfg.block_size} tokens "
                   f"({self.runner.storage.num_bytes() / 2**30:.2f} GiB), weights "
@@ -74,7 +74,7 @@ class LLMEngine:
             import warnings
             warnings.warn(f"{len(kept)} weight matrices are stored in float32 and stay so (first: {kept[0]}): their "
                           f"products run on the 32-bit kernels, much slower than bfloat16; save the checkpoint in "
-                          f"bfloat16 for speed", stacklevel=2)
+                          f"bfloat16, or set EngineConfig.cast_float32_weights, for speed", stacklevel=2)
         self.tokenizer = None
         if load_tokenizer and isinstance(model, str):
             from transformers import AutoTokenizer      # text in and out only; never on the token path
@@ -189,7 +189,7 @@ class LLMEngine:
             seq.token_ids[place] = tok
             if seq.first_token_time is None:
                 seq.first_token_time = now
-            stopped = tok == self.eos_token_id and not seq.params.ignore_eos
+            stopped = tok in self.stop_token_ids and not seq.params.ignore_eos
             if not (stopped or (seq.ending and place == seq.num_tokens - 1)):
                 continue
             del seq.token_ids[place + 1:]      # a placeholder of the row started meanwhile, if any
@@ -201,6 +201,16 @@ class LLMEngine:
                 seq.status = Status.FINISHED
             finished.append(seq)
         return finished
+
+    @property
+    def eos_token_id(self):
+        """The stop id, under the name the reference's engine has (inference_engine/engine.py:217); the first
+        one if the model has several.  Assigning replaces them all by one id."""
+        return min(self.stop_token_ids) if self.stop_token_ids else None
+
+    @eos_token_id.setter
+    def eos_token_id(self, token):
+        self.stop_token_ids = frozenset() if token is None else frozenset([int(token)])
 
     # --------------------------------------------------------------- offline
     def generate(self, prompts, params: SamplingParams | list | None = None, decode_text: bool = True

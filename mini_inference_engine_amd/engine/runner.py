@@ -32,7 +32,7 @@ class ModelRunner:
     def __init__(self, model, *, dtype=torch.bfloat16, device="cuda", backend=None, page_size: int = 16,
                  num_pages: int | None = None, memory_fraction: float = 0.85, reserve_bytes: int = 768 * 2**20,
                  max_step_tokens: int = 2048, max_rows: int = 256, max_model_len: int | None = None,
-                 num_state_slots: int | None = None, weights=None):
+                 num_state_slots: int | None = None, weights=None, cast_float32_weights: bool = False):
         """``model``: a folder with config.json and safetensors, or a ModelConfig together
         with ``weights`` (name -> tensor).  ``backend``: the kernels; by default the HIP
         library, which must load (there is no other product path)."""
@@ -52,7 +52,7 @@ class ModelRunner:
             backend = HipBackend(self.dtype, self.device)
         self.ops = backend
         self.model.use_backend(backend)
-        self.load_report = load_weights(self.model, source, self.device, self.dtype)
+        self.load_report = load_weights(self.model, source, self.device, self.dtype, cast_float32=cast_float32_weights)
         self.model.prepare(self.device, self.dtype)
 
         spec = self.model.spec

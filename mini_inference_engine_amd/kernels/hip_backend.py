@@ -490,14 +490,23 @@ class HipBackend(KernelBackend):
         """A step of single-token rows whose rows and kv heads alone fill the GPU: the decode kernel finishes the
         projection itself (no kernel between product and attention).  None: not such a step."""
         T = pending.part.shape[1]
+        # The kernel rotates with the step's positions, takes the row's own key from its LDS and writes it to
+        # pending.slots: that is the same result as finish() only if the projection was made for this very step
+        # and this page group (same position and slot arrays, same caches).  Anything else takes finish().
         if (forced or step.num_decode_rows != T or step.num_tokens != T or Hq // Hkv > 16
-                or pending.k_cache is not k_cache or pending.v_cache is not v_cache):
+                or pending.k_cache is not k_cache or pending.v_cache is not v_cache
+                or pending.positions.data_ptr() != step.positions.data_ptr()
+                or pending.slots.data_ptr() != group.slot_mapping.data_ptr()
+                or (pending.Hq, pending.Hkv, pending.D) != (Hq, Hkv, D)):
             return None
         lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))
         block_keys = lib.mie_decode_block_keys()
         partition, splits = self.decode_splits(T, Hq, Hkv, step.max_context, window, block_keys, D)
         if splits != 1:
             return None
+        bound = min(step.max_context, window + 32) if window else step.max_context
+        if partition < bound:
+            raise AssertionError(f"decode attention from sums: one split of {partition} keys for contexts up to {bound}")
         part = pending.part
         self._on_device(k_cache, v_cache)
         _, _, bt = self._check_attention_cache(T, torch.bfloat16, Hkv, D, k_cache, v_cache, group, step)

@@ -36,10 +36,38 @@ from typing import Any, Sequence
 
 @dataclass(frozen=True)
 class Source:
-    """One checkpoint tensor and where its rows go inside a (possibly fused) buffer."""
+    """One piece of a device buffer and the checkpoint tensor it comes from.
+
+    ``shape`` is the piece as it lands in the buffer, ``row_offset`` where its rows go inside a stacked buffer.
+    By default the piece is the whole checkpoint tensor ``name``.  A checkpoint that stores things differently
+    is declared, not special-cased in the loader:
+      stored_shape   shape of the checkpoint tensor, where it differs from ``shape``
+      rows, cols     (start, stop): the part of the stored tensor's dim 0 / dim 1 this piece takes (a fused
+                     tensor of the checkpoint split over several buffers; several Sources may name one tensor)
+      transform      name of a registered function (register_weight_transform) applied to the slice; its
+                     result must have ``shape`` ("transpose" ships: a matrix stored [in, out])
+    """
     name: str
     shape: tuple
     row_offset: int = 0
+    stored_shape: tuple | None = None
+    rows: tuple | None = None
+    cols: tuple | None = None
+    transform: str | None = None
+
+    @property
+    def checkpoint_shape(self) -> tuple:
+        return tuple(self.stored_shape) if self.stored_shape is not None else tuple(self.shape)
+
+
+# name -> function(tensor) -> tensor, applied by the loader to a Source's slice of its checkpoint tensor
+WEIGHT_TRANSFORMS: dict = {"transpose": lambda t: t.t()}
+
+
+def register_weight_transform(name: str, fn) -> None:
+    """A way a checkpoint stores a tensor differently from how a part wants it (per-head interleaving, [in, out]
+    matrices, ...), by name, so that a part can ask for it in a Source from outside the package too."""
+    WEIGHT_TRANSFORMS[name] = fn
 
 
 @dataclass(frozen=True)
@@ -49,23 +77,29 @@ class ParamSpec:
     shape: tuple
     sources: tuple
     integer: bool = False   # integer tables are kept as int32
-    init: str = "weight"    # how the random-weights mode draws it: "weight" N(0, std), "scale" 1 + N(0, std), "zeros"
+    init: str = "weight"    # how the random-weights mode draws it: "weight" N(0, std), "scale" 1 + N(0, std), "zeros";
+                            # integer tables: uniform in [0, integer_bound)
+    integer_bound: int = 0  # random-weights mode: an integer table's entries are drawn below this
 
     @staticmethod
-    def single(attr: str, name: str, shape: Sequence[int], integer: bool = False, init: str = "weight") -> "ParamSpec":
+    def single(attr: str, name: str, shape: Sequence[int], integer: bool = False, init: str = "weight",
+               integer_bound: int = 0) -> "ParamSpec":
         shape = tuple(int(s) for s in shape)
-        return ParamSpec(attr, shape, (Source(name, shape, 0),), integer, init)
+        return ParamSpec(attr, shape, (Source(name, shape, 0),), integer, init, integer_bound)
 
     @staticmethod
-    def stacked(attr: str, pieces: Sequence[tuple]) -> "ParamSpec":
-        """pieces: (name, shape) in row order; all share the trailing dims."""
+    def stacked(attr: str, pieces: Sequence) -> "ParamSpec":
+        """pieces, in row order: (name, shape) for a whole checkpoint tensor, or a Source (whose row_offset is
+        set here) for a slice or a transformed tensor; all share the trailing dims."""
         sources, off = [], 0
-        tail = tuple(pieces[0][1][1:])
-        for name, shape in pieces:
-            shape = tuple(int(s) for s in shape)
+        first = pieces[0]
+        tail = tuple((first.shape if isinstance(first, Source) else first[1])[1:])
+        for piece in pieces:
+            src = piece if isinstance(piece, Source) else Source(piece[0], tuple(int(s) for s in piece[1]))
+            shape = tuple(int(s) for s in src.shape)
             if tuple(shape[1:]) != tail:
-                raise ValueError(f"cannot stack {name} {shape} on tail {tail}")
-            sources.append(Source(name, shape, off))
+                raise ValueError(f"cannot stack {src.name} {shape} on tail {tail}")
+            sources.append(Source(src.name, shape, off, src.stored_shape, src.rows, src.cols, src.transform))
             off += shape[0]
         return ParamSpec(attr, (off,) + tail, tuple(sources))
 
@@ -278,7 +312,7 @@ class DecoderSpec:
     head: Part
     schedule: list = field(default_factory=list)
     ignore_tensors: tuple = ()      # regular expressions of checkpoint names to skip
-    eos_token_id: int | None = None
+    stop_token_ids: tuple = ()      # a request ends when it draws one of these (unless told to ignore them)
     max_position: int | None = None
     vocab_size: int = 0
 

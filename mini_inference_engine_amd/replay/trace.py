@@ -1,6 +1,6 @@
 """Trace replay: feed given token ids through the model step by step, write logits.
 
-    trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+    trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--max-requests R]
 
 Steps come on standard input, one JSON object a line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
@@ -30,6 +30,9 @@ def _parser():
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time, each request's count rounded up to a "
                          "multiple of 64 (or of the page size if that is larger); sizes the page pool")
+    ap.add_argument("--max-requests", type=int, default=4,
+                    help="most requests live at a time (default 4); a trace with more is refused at the step that "
+                         "opens one too many")
     ap.add_argument("--hip-graphs", action="store_true",
                     help="run steps of single-token entries through captured graphs, as generation does")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
@@ -37,8 +40,9 @@ def _parser():
     return ap
 
 
-def replay(runner, lines, out_dir: str, say=print) -> int:
-    """Runs the steps in ``lines`` on ``runner``.  Returns the number of steps."""
+def replay(runner, lines, out_dir: str, say=print, max_live: int | None = None) -> int:
+    """Runs the steps in ``lines`` on ``runner``.  Returns the number of steps.  ``max_live``: the most
+    requests that may be live at a time (the page pool was sized for that many); one more is an error."""
     import numpy as np
     from ..engine.batch import StepRow
 
@@ -60,6 +64,9 @@ def replay(runner, lines, out_dir: str, say=print) -> int:
             if bad:
                 raise ValueError(f"step {step_no}: token ids outside the vocabulary: {bad[:5]}")
             if rid not in live:
+                if max_live is not None and len(live) >= max_live:
+                    raise RuntimeError(f"step {step_no}: request {rid!r} would be live beside {len(live)} others; the "
+                                       f"page pool was made for {max_live} (--max-requests)")
                 live[rid] = [runner.cache.open(rid), 0]
             rc, have = live[rid]
             if not runner.cache.reserve(rc, have, len(toks)):
@@ -88,19 +95,20 @@ def replay(runner, lines, out_dir: str, say=print) -> int:
 def main(argv=None) -> int:
     args = _parser().parse_args(argv)
     from ..engine.runner import ModelRunner
-    page = args.block_size
+    page, live = args.block_size, max(1, args.max_requests)
     # --max-tokens counts every live request rounded up to 64 tokens, so whole pages cover it; a page more for each
-    # of the four requests that may be live keeps a count that was not rounded from running out, + the scratch page
-    pages = -(-args.max_tokens // page) + 4 + 1
+    # request that may be live keeps a count that was not rounded from running out (a request wastes less than a
+    # page), + the scratch page
+    pages = -(-args.max_tokens // page) + live + 1
     runner = ModelRunner(args.model, dtype=args.dtype, device=args.device, page_size=page, num_pages=pages,
-                         max_step_tokens=max(64, args.max_tokens), max_rows=64)
+                         max_step_tokens=max(64, args.max_tokens), max_rows=live)
     if args.hip_graphs:
-        runner.capture_decode_graphs((1, 2, 4, 8))
+        runner.capture_decode_graphs(tuple(b for b in (1, 2, 4, 8, 16, 32, 64) if b < 2 * live))
 
     def say(msg):
         print(msg, flush=True)
 
-    replay(runner, sys.stdin, args.out, say)
+    replay(runner, sys.stdin, args.out, say, max_live=live)
     return 0
 
 

@@ -7,9 +7,14 @@ silently.  Here every problem of a checkpoint is collected and raised as one
 WeightError that lists missing tensors, unexpected tensors and wrong shapes.
 
 Dtypes: in bfloat16 mode a tensor stored in bfloat16 (or float16) is kept in
-bfloat16 and a tensor stored in 32-bit stays 32-bit; integer tables become
-int32.  In float32 mode every float tensor is widened to float32.  Fused buffers
-(q,k,v rows; gate,up rows) are filled piece by piece, straight from the file.
+bfloat16 and a tensor stored in 32-bit stays 32-bit (``cast_float32=True``
+rounds those to bfloat16 too, as the reference does with every tensor,
+inference_engine/model.py:94); integer tables become int32.  In float32 mode
+every float tensor is widened to float32.  Fused buffers (q,k,v rows; gate,up
+rows) are filled piece by piece, straight from the file.  A piece is a whole
+checkpoint tensor, or rows / columns of one, optionally passed through a named
+transform (parts.base.Source): how a checkpoint stores a tensor is declared by
+the part, the loader knows no model.
 """
 from __future__ import annotations
 
@@ -72,8 +77,12 @@ class CheckpointFiles:
     def shape(self, name: str) -> tuple:
         return tuple(self._handles[self.where[name]].get_slice(name).get_shape())
 
-    def tensor(self, name: str) -> torch.Tensor:
-        return self._handles[self.where[name]].get_tensor(name)
+    def tensor(self, name: str, rows=None) -> torch.Tensor:
+        """The tensor, or rows [start, stop) of it, read from the file without the rest."""
+        h = self._handles[self.where[name]]
+        if rows is None:
+            return h.get_tensor(name)
+        return h.get_slice(name)[rows[0]:rows[1]]
 
 
 class TensorDict:
@@ -89,8 +98,9 @@ class TensorDict:
     def shape(self, name):
         return tuple(self.tensors[name].shape)
 
-    def tensor(self, name):
-        return self.tensors[name]
+    def tensor(self, name, rows=None):
+        t = self.tensors[name]
+        return t if rows is None else t[rows[0]:rows[1]]
 
 
 _FLOATS = (torch.float32, torch.bfloat16, torch.float16, torch.float64)
@@ -106,7 +116,23 @@ def storage_dtype(stored: torch.dtype, mode: torch.dtype, integer: bool) -> torc
     return torch.float32 if stored in (torch.float32, torch.float64) else torch.bfloat16
 
 
-def load_weights(model, source, device, mode: torch.dtype) -> dict:
+def _piece(source, s):
+    """The part of checkpoint tensor ``s.name`` that Source ``s`` asks for, sliced and transformed."""
+    from ..parts.base import WEIGHT_TRANSFORMS
+    t = source.tensor(s.name, s.rows) if s.rows is not None else source.tensor(s.name)
+    if s.cols is not None:
+        t = t[:, s.cols[0]:s.cols[1]]
+    if s.transform is not None:
+        if s.transform not in WEIGHT_TRANSFORMS:
+            raise KeyError(f"{s.name}: weight transform {s.transform!r} is not registered (known: {sorted(WEIGHT_TRANSFORMS)})")
+        t = WEIGHT_TRANSFORMS[s.transform](t)
+    if tuple(t.shape) != tuple(s.shape):
+        raise ValueError(f"{s.name}: rows {s.rows}, columns {s.cols}, transform {s.transform!r} of the stored tensor give "
+                         f"{tuple(t.shape)}; the part declared {tuple(s.shape)}")
+    return t
+
+
+def load_weights(model, source, device, mode: torch.dtype, cast_float32: bool = False) -> dict:
     """Fill every declared buffer of ``model`` (a Decoder) from ``source`` (folder
     path, CheckpointFiles or name -> tensor dict).  Returns a small report."""
     if isinstance(source, str):
@@ -114,25 +140,28 @@ def load_weights(model, source, device, mode: torch.dtype) -> dict:
     elif isinstance(source, dict):
         source = TensorDict(source)
     specs = model.param_specs()
-    wanted = {}
+    wanted, clash = {}, []
     for part, spec in specs:
         for s in spec.sources:
-            wanted.setdefault(s.name, s.shape)
+            if wanted.setdefault(s.name, s.checkpoint_shape) != s.checkpoint_shape:
+                clash.append(f"parts disagree about the stored shape of {s.name}: {wanted[s.name]} and {s.checkpoint_shape}")
     present = set(source.names())
     ignore = [re.compile(p) for p in model.spec.ignore_tensors]
     missing = sorted(n for n in wanted if n not in present)
     unexpected = sorted(n for n in present if n not in wanted and not any(r.fullmatch(n) for r in ignore))
     wrong = [(n, source.shape(n), wanted[n]) for n in sorted(wanted) if n in present
              and tuple(source.shape(n)) != tuple(wanted[n])]
-    if missing or unexpected or wrong:
-        raise WeightError(source.folder, missing, unexpected, wrong)
+    if missing or unexpected or wrong or clash:
+        raise WeightError(source.folder, missing, unexpected, wrong, clash)
 
     ignored = sorted(n for n in present if n not in wanted)
     kept_float32 = []
     for part, spec in specs:
-        pieces = [source.tensor(s.name) for s in spec.sources]
+        pieces = [_piece(source, s) for s in spec.sources]
         kinds = {storage_dtype(t.dtype, mode, spec.integer) for t in pieces}
         dtype = torch.float32 if torch.float32 in kinds else kinds.pop()
+        if dtype == torch.float32 and mode != torch.float32 and cast_float32:
+            dtype = mode
         if dtype == torch.float32 and mode != torch.float32 and len(spec.shape) >= 2:
             # kept as stored; the products of this matrix then run on the 32-bit kernels, far slower than the
             # bfloat16 ones: worth a line, since a checkpoint saved in float32 does this to every layer

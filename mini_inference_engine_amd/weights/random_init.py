@@ -4,7 +4,10 @@ through the same loader a real checkpoint does.
 
 Matrices and embeddings are N(0, std), vectors (norm weights) 1 + N(0, std),
 drawn in float32 from one seeded CPU generator in the order the parts declare
-their tensors, then stored in the asked dtype.
+their tensors, then stored in the asked dtype; integer tables are uniform below
+the bound their part declares and stored as int32.  What is drawn is the tensor
+as the checkpoint stores it (a part may take rows or columns of it, or a
+transform of it).
 """
 from __future__ import annotations
 
@@ -29,10 +32,14 @@ def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std: 
             if s.name in out:
                 continue
             if spec.integer:
-                raise NotImplementedError("random integer tables")
+                if spec.integer_bound < 1:
+                    raise ValueError(f"{s.name}: an integer table needs integer_bound >= 1 to be drawn at random")
+                out[s.name] = torch.randint(0, spec.integer_bound, s.checkpoint_shape, generator=gen, dtype=torch.int32,
+                                            device=device)
+                continue
             # every tensor draws from the generator, whatever its kind, so that adding a part does not shift
             # the values of the parts after it
-            t = torch.randn(s.shape, generator=gen, dtype=torch.float32, device=device) * std
+            t = torch.randn(s.checkpoint_shape, generator=gen, dtype=torch.float32, device=device) * std
             if spec.init == "scale":
                 t = t + 1.0
             elif spec.init == "zeros":

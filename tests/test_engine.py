@@ -110,6 +110,23 @@ def test_eos_stops_and_stays(tiny_models):
     assert out[0].output_ids == toks[:stop + 1], "generation ends with the stop token, which stays in the output"
 
 
+def test_every_stop_id_of_the_configuration_stops(tiny_models):
+    """config.json may list several stop ids; each of them ends a request (the reference keeps the first only)."""
+    from mini_inference_engine_amd.config import LlamaConfig
+    m = tiny_models["A"]
+    prompts = prompts_for(m, [12], seed=6)
+    toks = engine(m, "cpu", "float32", num_blocks=16).generate(prompts, SamplingParams(max_tokens=20, ignore_eos=True))[0].output_ids
+    first = [i for i, t in enumerate(toks) if t not in toks[:i]]      # places where a token appears for the first time
+    stop_at, later = first[2], first[-1]
+    early, late = toks[stop_at], toks[later]
+    assert stop_at < later
+    config = LlamaConfig.from_dict({**m["cfg"], "eos_token_id": [late, early]})
+    eng = LLMEngine(config, EngineConfig(num_blocks=16), dtype="float32", device="cpu", backend=TorchBackend(torch.float32),
+                    weights=m["weights"], verbose=False)
+    assert eng.stop_token_ids == {late, early}
+    assert eng.generate(prompts, SamplingParams(max_tokens=20))[0].output_ids == toks[:stop_at + 1]
+
+
 def test_running_a_step_ahead_changes_no_token(tiny_models):
     """A step is started before the host has read the tokens of the one before (the device hands them on);
     stop tokens are then seen a step late.  Tokens, ends and the cache's books must be what they are when

@@ -146,7 +146,7 @@ def build_toy(cfg: ToyConfig) -> DecoderSpec:
     emb = Embedding(cfg.vocab, w, "emb")
     return DecoderSpec(embedding=emb, layers=layers, final_norm=norm("out_norm"), head=LMHead(cfg.vocab, w, "head", emb),
                        schedule=[LayerCall(0), LayerCall(1), LayerCall(2), LayerCall(1), LayerCall(3, cache_of=2)],
-                       max_position=256, vocab_size=cfg.vocab, eos_token_id=None)
+                       max_position=256, vocab_size=cfg.vocab, stop_token_ids=())
 
 
 @pytest.fixture(scope="module")
@@ -372,7 +372,7 @@ def build_routed(cfg: RoutedConfig) -> DecoderSpec:
               for i in range(2)]
     emb = Embedding(cfg.vocab, w, "emb")
     return DecoderSpec(embedding=emb, layers=layers, final_norm=RMSNorm(w, 1e-5, "out_norm"),
-                       head=LMHead(cfg.vocab, w, "head", emb), max_position=256, vocab_size=cfg.vocab, eos_token_id=None)
+                       head=LMHead(cfg.vocab, w, "head", emb), max_position=256, vocab_size=cfg.vocab, stop_token_ids=())
 
 
 @pytest.fixture(scope="module")

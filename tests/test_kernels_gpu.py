@@ -695,6 +695,7 @@ def test_decode_attention_finishes_the_projection(engine_ops, geom, window):
     pos = step.positions
     bt = group.block_tables
     slots = (bt[torch.arange(M, device=DEV), (pos // page).long()] * page + pos % page).to(torch.int32)
+    group.slot_mapping = slots
     scale = 0.9 / math.sqrt(D)
 
     kc1, vc1 = kc.clone(), vc.clone()
@@ -715,6 +716,14 @@ def test_decode_attention_finishes_the_projection(engine_ops, geom, window):
     # and against the exact attention over that cache
     expect = ref.ref_paged_attention(q2, Hq, Hkv, D, kc2, vc2, bt, step.token_row, pos, scale, window, torch.float64)
     torch.testing.assert_close(out1.double(), expect, **ATT_TOL[torch.bfloat16])
+    # a projection that was made for other positions or slots than the step's is finished in a kernel of its own
+    # (with its own positions and slots), not by the attention kernel (which would use the step's)
+    kc4, vc4 = kc.clone(), vc.clone()
+    pending = o.linear_rotary_kv_store(x, w, pos.clone(), cos, sin, D, Hq, Hkv, D, kc4, vc4, slots, for_attention=True)
+    assert o._decode_attention_from_sums(pending, Hq, Hkv, D, kc4, vc4, group, step, scale, window, False) is None
+    pending = o.linear_rotary_kv_store(x, w, pos, cos, sin, D, Hq, Hkv, D, kc4, vc4, slots.clone(), for_attention=True)
+    assert o._decode_attention_from_sums(pending, Hq, Hkv, D, kc4, vc4, group, step, scale, window, False) is None
+    assert torch.equal(kc4, kc), "a refused step writes nothing"
     # a step that is not of this kind finishes the projection in a kernel of its own
     kc3, vc3 = kc.clone(), vc.clone()
     pending = o.linear_rotary_kv_store(x, w, pos, cos, sin, D, Hq, Hkv, D, kc3, vc3, slots, for_attention=True)

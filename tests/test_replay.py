@@ -175,3 +175,37 @@ def test_trace_run_program(tiny_models, tmp_path, dtype, graphs):
     got = trace_util.read_outputs(out, steps, 256)
     exp = expected_logits(m, prompts, bf16_weights=dtype == "bfloat16")
     trace_util.compare(got, exp, F32_TOL if dtype == "float32" else BF16_TOL, f"trace_run/{dtype}")
+
+
+def test_replay_refuses_one_request_too_many(tiny_models, tmp_path):
+    m = tiny_models["A"]
+    prompts = trace_util.random_prompts(256, [20, 21, 22], seed=3)
+    steps = trace_util.mixed(prompts, max_live=3, seed=2, tail=4)
+    runner = ModelRunner(m["config"], weights=m["weights"], dtype="float32", device="cpu",
+                         backend=TorchBackend(torch.float32), num_pages=12, max_rows=4, max_step_tokens=64)
+    with pytest.raises(RuntimeError, match="--max-requests"):
+        replay(runner, trace_util.to_lines(steps), str(tmp_path), lambda s: None, max_live=2)
+
+
+@pytest.mark.gpu
+def test_trace_run_program_with_six_live_requests_and_the_true_peak(tiny_models, tmp_path):
+    """More live requests than the default four, lengths that are no multiple of a page, and --max-tokens the
+    true peak of live tokens, not rounded up per request: --max-requests sizes the pool's slack."""
+    m = tiny_models["B"]
+    lengths = [33, 17, 50, 21, 45, 39, 27, 61, 19]
+    prompts = trace_util.random_prompts(384, lengths, seed=8)
+    steps = trace_util.mixed(prompts, max_live=6, seed=4, tail=5)
+    assert max(len(s["entries"]) for s in steps) >= 5
+    true_peak = trace_util.live_token_peak(steps, round_to=1)
+    assert true_peak < trace_util.live_token_peak(steps) and true_peak % 16
+    out = str(tmp_path / "out")
+    base = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", m["folder_bf16"], "--dtype", "bfloat16",
+            "--out", out, "--max-tokens", str(true_peak)]
+    text = "\n".join(trace_util.to_lines(steps)) + "\n"
+    proc = subprocess.run(base + ["--max-requests", "6"], input=text, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = trace_util.read_outputs(out, steps, 384)
+    trace_util.compare(got, expected_logits(m, prompts, bf16_weights=True), BF16_TOL, "trace_run/six live")
+    # without the option the fifth live request is refused by name, not by running out of pages somewhere
+    proc = subprocess.run(base, input=text, capture_output=True, text=True, timeout=600)
+    assert proc.returncode != 0 and "--max-requests" in proc.stderr
