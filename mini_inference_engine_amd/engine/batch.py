@@ -51,6 +51,9 @@ class StepContext:
     state_slots: torch.Tensor        # [rows] int32
     logit_rows: torch.Tensor         # [num_logits] int32 flat token positions, in the caller's order
     taken_from: torch.Tensor | None = None      # [T] int32, see StepRow.taken_from; -1 where input_ids holds the token
+    sample_temps: torch.Tensor | None = None    # [num_logits] float32: temperature of each wanted row (0 = greedy), if
+    sample_seeds: torch.Tensor | None = None    # [num_logits] int64    the step's caller wants tokens chosen from its
+    sample_counters: torch.Tensor | None = None  # [num_logits] int32   logits (seed and output index of the noise stream)
     earlier_tokens: torch.Tensor | None = None  # int32: the tokens the last step chose (set by the runner)
     groups: list = field(default_factory=list)
     page_size: int = 0
@@ -67,7 +70,9 @@ class StepArena:
         self.device = torch.device(device)
         fields_ = [("input_ids", max_tokens), ("taken_from", max_tokens), ("positions", max_tokens), ("token_row", max_tokens),
                    ("logit_rows", max_tokens), ("row_start", max_rows + 1), ("row_position", max_rows),
-                   ("row_context", max_rows), ("state_slots", max_rows)]
+                   ("row_context", max_rows), ("state_slots", max_rows),
+                   # what choosing a token from a row's logits needs: they travel with the step's other arrays
+                   ("sample_temps", max_rows), ("sample_counters", max_rows), ("sample_seeds", 2 * max_rows)]
         for g in range(num_groups):
             fields_.append((f"slot_mapping{g}", max_tokens))
         for g in range(num_groups):
@@ -117,10 +122,13 @@ def order_rows(rows: Sequence[StepRow]) -> list[int]:
 
 
 def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad_rows_to: int = 0,
-               static_context: int = 0, want_all: bool = False) -> StepContext:
+               static_context: int = 0, want_all: bool = False, sampling=None) -> StepContext:
     """Flatten ``rows`` into ``arena``.  ``pad_rows_to`` adds scratch rows (one token at
     position 0, page 0, slot 0) up to a captured batch size.  ``want_all`` asks for the logits
-    of every token in flat order (what a captured step produces) instead of the rows' wants."""
+    of every token in flat order (what a captured step produces) instead of the rows' wants.
+    ``sampling``: (temperatures, seeds, counters), one entry for each wanted row of logits in their order
+    (with ``want_all``: one for each of ``rows``; scratch rows are greedy), for a step whose tokens are
+    chosen on the device."""
     arena.wait_uploaded()           # the last step's copy may still be reading the host mirror
     order = order_rows(rows)
     n_rows = len(rows)
@@ -186,6 +194,17 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
             wanted.append(base + w)
     R = len(wanted)
     arena.host_view("logit_rows")[:R] = wanted
+    if sampling is not None:
+        temps, seeds, counters = sampling
+        n = len(temps)
+        if not (len(seeds) == len(counters) == n) or n != (n_rows if want_all else R) or R > arena.max_rows:
+            raise ValueError(f"sampling inputs for {n} rows; the step has {n_rows if want_all else R} rows of wanted "
+                             f"logits (at most {arena.max_rows})")
+        ht, hc, hs = arena.host_view("sample_temps"), arena.host_view("sample_counters"), arena.host_view("sample_seeds")
+        ht[:R], hc[:R], hs[:2 * R] = 0, 0, 0
+        ht[:n] = np.asarray(temps, dtype=np.float32).view(np.int32)
+        hc[:n] = np.asarray(counters, dtype=np.int32)
+        hs[:2 * n] = np.asarray([s & 0xFFFFFFFFFFFFFFFF for s in seeds], dtype=np.uint64).view(np.int32)
 
     mb = arena.max_blocks
     for g in range(arena.num_groups):
@@ -216,6 +235,10 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
         host={"row_start": row_start, "row_position": row_pos, "row_context": ctx, "row_len": row_len,
               "positions": positions, "token_row": token_row, "state_slots": slots_state[:total_rows].copy()},
     )
+    if sampling is not None:
+        step.sample_temps = arena.dev_view("sample_temps", R).view(torch.float32)
+        step.sample_counters = arena.dev_view("sample_counters", R)
+        step.sample_seeds = arena.dev_view("sample_seeds", 2 * R).view(torch.int64)
     for g in range(arena.num_groups):
         step.groups.append(GroupStep(
             block_tables=arena.dev_view(f"block_tables{g}", total_rows * mb).view(total_rows, mb),

@@ -17,7 +17,7 @@ import torch
 
 
 class DecodeGraphs:
-    def __init__(self, runner, batch_sizes, verbose: bool = True):
+    def __init__(self, runner, batch_sizes, verbose: bool = True, sample: bool = False):
         # The runner owns this object, so it is not kept here: a reference back would make a cycle, and the
         # graphs with all they hold would then be freed whenever the collector runs, possibly in the middle
         # of a later capture, which the runtime does not survive.  ``run`` takes the runner instead.
@@ -25,13 +25,15 @@ class DecodeGraphs:
         self.sizes = sorted(b for b in set(batch_sizes) if 0 < b <= arena.max_rows and b <= arena.max_tokens)
         self.graphs = {}
         self.static_context = runner.max_model_len
+        self.sample = sample               # the captured step also chooses a token from every row's logits
         if not self.sizes:
             return
         t0 = time.perf_counter()
         pool = None
         for bs in reversed(self.sizes):                 # largest first: smaller ones reuse its pool
-            step = runner.build([], pad_rows_to=bs, static_context=self.static_context, want_all=True)
-            runner.model.forward(step)                  # loads libraries, warms the allocator
+            step = runner.build([], pad_rows_to=bs, static_context=self.static_context, want_all=True,
+                                sampling=([], [], []) if sample else None)
+            self._forward(runner, step, bs)             # loads libraries, warms the allocator
             torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
             # no garbage collection while the stream records: a collected object that owns device memory
@@ -40,7 +42,7 @@ class DecodeGraphs:
             gc.disable()
             try:
                 with torch.cuda.graph(g, pool=pool):
-                    logits = runner.model.forward(step)
+                    logits = self._forward(runner, step, bs)
             finally:
                 if collecting:
                     gc.enable()
@@ -51,18 +53,29 @@ class DecodeGraphs:
             print(f"[mini_inference_engine_amd] captured {len(self.sizes)} decode graphs "
                   f"(batch <= {self.sizes[-1]}) in {time.perf_counter() - t0:.1f} s", flush=True)
 
+    def _forward(self, runner, step, bs):
+        logits = runner.model.forward(step)
+        if self.sample:
+            runner.ops.sample(logits, step.sample_temps, step.sample_seeds, step.sample_counters,
+                              out=runner.chosen_tokens[:bs])
+        return logits
+
     def fits(self, rows: int) -> bool:
         return bool(self.sizes) and rows <= self.sizes[-1]
 
-    def run(self, runner, rows) -> torch.Tensor | None:
-        """``rows``: single-token StepRows.  Logits of the rows that want them, in order."""
+    def run(self, runner, rows, sampling=None):
+        """``rows``: single-token StepRows.  Logits of the rows that want them, in order, and the step as
+        built.  ``sampling`` (one entry a row): with graphs that sample, row i's token is in
+        ``runner.chosen_tokens[i]`` afterwards."""
         bs = next(s for s in self.sizes if s >= len(rows))
         picked = [i for i, r in enumerate(rows) if len(r.want)]
-        runner.build(rows, pad_rows_to=bs, static_context=self.static_context, want_all=True)
+        if sampling is None and self.sample:
+            sampling = ([0.0] * len(rows), [0] * len(rows), [0] * len(rows))     # nobody reads what is chosen
+        step = runner.build(rows, pad_rows_to=bs, static_context=self.static_context, want_all=True, sampling=sampling)
         g, logits = self.graphs[bs]
         g.replay()
         if not picked:
-            return None
+            return None, step
         if len(picked) == len(rows):
-            return logits[:len(rows)]
-        return logits[torch.tensor(picked, device=logits.device)]
+            return logits[:len(rows)], step
+        return logits[torch.tensor(picked, device=logits.device)], step

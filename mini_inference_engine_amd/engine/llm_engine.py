@@ -62,7 +62,7 @@ class LLMEngine:
         if cfg.poison_freed_pages:
             self.cache.on_release = self.runner.storage.poison_pages
         self.scheduler = Scheduler(self.cfg, self.cache)
-        self.sampler = Sampler(self.runner.ops, self.runner.device, cfg.max_num_seqs, out=self.runner.chosen_tokens)
+        self.sampler = Sampler(self.runner.device, cfg.max_num_seqs, out=self.runner.chosen_tokens)
         self._in_flight = None             # the step whose tokens the host has not read yet
         self.stop_token_ids = frozenset(self.runner.model.spec.stop_token_ids)
         if verbose:
@@ -80,7 +80,7 @@ class LLMEngine:
             from transformers import AutoTokenizer      # text in and out only; never on the token path
             self.tokenizer = AutoTokenizer.from_pretrained(model)
         if cfg.use_hip_graphs and self.runner.device.type == "cuda":
-            self.runner.capture_decode_graphs(cfg.graph_batch_sizes, verbose=verbose)
+            self.runner.capture_decode_graphs(cfg.graph_batch_sizes, verbose=verbose, sample=True)
         self.graphs = self.runner.graphs
         self.num_steps = 0
         self.num_graph_steps = 0
@@ -158,15 +158,11 @@ class LLMEngine:
             if last:
                 sample_seqs.append(seq)
 
-        logits = self.runner.forward_step(rows)       # a captured graph when every row is a single token
+        # a captured graph when every row is a single token; the tokens are chosen in the step as well
+        self.runner.forward_step(rows, sampling=self.sampler.sampling_inputs(sample_seqs) if sample_seqs else None)
         self.num_steps += 1
         self.num_graph_steps += self.runner.last_step_captured
-
-        chosen = None
-        if sample_seqs:
-            chosen = self.sampler.sample_async(
-                logits, [s.params.temperature for s in sample_seqs], [s.seed for s in sample_seqs],
-                [s.num_output_tokens for s in sample_seqs])
+        chosen = self.sampler.fetch_async(len(sample_seqs)) if sample_seqs else None
 
         # what is certain whatever the tokens turn out to be
         for seq, n in batch:

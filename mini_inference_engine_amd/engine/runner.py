@@ -99,23 +99,39 @@ class ModelRunner:
         step.earlier_tokens = self.chosen_tokens
         return step
 
-    def capture_decode_graphs(self, batch_sizes, verbose: bool = False) -> None:
+    def capture_decode_graphs(self, batch_sizes, verbose: bool = False, sample: bool = False) -> None:
         """Capture the forward of a step of single-token rows once per batch size; ``forward_step``
         then replays the smallest captured size that holds such a step instead of launching kernel by
-        kernel (inference_engine/engine.py:76-120)."""
+        kernel (inference_engine/engine.py:76-120).  ``sample``: the captured step also chooses a token
+        from every row's logits (for callers that pass ``sampling`` to ``forward_step``)."""
         from .graphs import DecodeGraphs
-        self.graphs = DecodeGraphs(self, batch_sizes, verbose=verbose)
+        self.graphs = DecodeGraphs(self, batch_sizes, verbose=verbose, sample=sample)
 
     @torch.inference_mode()
-    def forward_step(self, rows: list[StepRow]) -> torch.Tensor | None:
+    def forward_step(self, rows: list[StepRow], sampling=None) -> torch.Tensor | None:
         """Logits [sum of wants, vocab] float32, ordered by row then by ``want``.
-        Pages for the rows' tokens must have been reserved."""
+        Pages for the rows' tokens must have been reserved.
+
+        ``sampling``: (temperatures, seeds, counters), one entry for each wanted row of logits: the step also
+        chooses a token from each of them on the device (temperature 0: the largest logit; else a draw whose
+        noise is a function of seed and counter) and leaves it in ``chosen_tokens[i]``.  The three arrays
+        travel with the step's other arrays, and in a captured step the choice is part of the graph."""
         self.last_step_captured = False
-        if self.graphs is not None and self.graphs.fits(len(rows)) and all(len(r.tokens) == 1 for r in rows):
+        captured = (self.graphs is not None and self.graphs.fits(len(rows)) and all(len(r.tokens) == 1 for r in rows)
+                    and (sampling is None or all(len(r.want) == 1 for r in rows)))
+        if captured:
             self.last_step_captured = True
-            return self.graphs.run(self, rows)
-        step = self.build(rows)
-        return self.model.forward(step)
+            logits, step = self.graphs.run(self, rows, sampling)
+            if sampling is None or self.graphs.sample:
+                return logits
+        else:
+            step = self.build(rows, sampling=sampling)
+            logits = self.model.forward(step)
+        if sampling is not None and logits is not None:
+            n = logits.shape[0]
+            self.ops.sample(logits, step.sample_temps[:n], step.sample_seeds[:n], step.sample_counters[:n],
+                            out=self.chosen_tokens[:n])
+        return logits
 
     def after_step(self, rows: list[StepRow]) -> None:
         """Tell the cache how far each row's request has come (windows release pages)."""

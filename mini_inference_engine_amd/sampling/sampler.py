@@ -10,7 +10,6 @@ and sampled rows alike with no host-side branch on the temperatures.
 """
 from __future__ import annotations
 
-import numpy as np
 import torch
 
 
@@ -29,55 +28,37 @@ class ChosenTokens:
 
 
 class Sampler:
-    def __init__(self, ops, device, max_rows: int, out: torch.Tensor | None = None):
-        """``out``: int32 device buffer of at least ``max_rows`` entries the chosen tokens are written
-        to (a fixed address a later step can read them from); by default one is made here."""
-        self.ops = ops
+    """Brings the tokens a step chose to the host.  The choice itself happens in the step (the runner's
+    ``forward_step(rows, sampling=...)``: its inputs travel with the step's other arrays, and a captured step
+    chooses inside its graph); ``sampling_inputs`` makes those inputs from the requests."""
+
+    def __init__(self, device, max_rows: int, out: torch.Tensor):
+        """``out``: the int32 device buffer the chosen tokens are written to (a fixed address a later step
+        can read them from)."""
         self.device = torch.device(device)
         pin = self.device.type == "cuda"
-        # one staging buffer: temperatures (float32 bits), counters, seeds (2 x int32 each)
-        self.host = torch.zeros(4 * max_rows, dtype=torch.int32, pin_memory=pin)
-        self.host_np = self.host.numpy()
-        self.dev = torch.zeros(4 * max_rows, dtype=torch.int32, device=self.device) if pin else self.host
         self.max_rows = max_rows
-        self.out = out if out is not None else torch.zeros(max(1, max_rows), dtype=torch.int32, device=self.device)
+        self.out = out
         # the chosen tokens travel to one of two pinned buffers in turn: the host may still be reading the
         # last step's while this step's copy is queued
         self._landing = [torch.zeros(max(1, max_rows), dtype=torch.int32, pin_memory=pin) for _ in range(2)]
         self._turn = 0
-        self._params_copied = None
 
-    def sample_async(self, logits: torch.Tensor, temperatures, seeds, counters) -> ChosenTokens:
-        """logits [R, V] float32; python lists of length R.  The tokens are written to ``self.out[:R]``
-        and copied towards the host; nothing is waited for."""
-        R = logits.shape[0]
-        if R > self.max_rows:
-            raise ValueError(f"{R} rows to sample, room for {self.max_rows}")
-        if self._params_copied is not None:
-            self._params_copied.synchronize()        # the staging buffer is free again
-        h = self.host_np
-        h[:R] = np.asarray(temperatures, dtype=np.float32).view(np.int32)
-        h[R:2 * R] = np.asarray(counters, dtype=np.int32)
-        h[2 * R:4 * R] = np.asarray([s & 0xFFFFFFFFFFFFFFFF for s in seeds], dtype=np.uint64).view(np.int32)
-        if self.dev is not self.host:
-            self.dev[:4 * R].copy_(self.host[:4 * R], non_blocking=True)
-            self._params_copied = torch.cuda.Event()
-            self._params_copied.record()
-        temps = self.dev[:R].view(torch.float32)
-        ctr = self.dev[R:2 * R]
-        sd = self.dev[2 * R:4 * R].view(torch.int64)
-        self.ops.sample(logits, temps, sd, ctr, out=self.out[:R])
-        if self.dev is self.host:               # no device: everything has happened already; keep a copy, since
-            return ChosenTokens(self.out[:R].clone(), None, R, None)     # the next step writes to ``out`` again
+    @staticmethod
+    def sampling_inputs(seqs):
+        """(temperatures, seeds, counters) of the requests a token is chosen for: the counter is the index of the
+        output token, so a request's draws do not depend on how it was batched, cut or preempted."""
+        return ([s.params.temperature for s in seqs], [s.seed for s in seqs], [s.num_output_tokens for s in seqs])
+
+    def fetch_async(self, count: int) -> ChosenTokens:
+        """The first ``count`` chosen tokens on their way to the host; nothing is waited for."""
+        if count > self.max_rows:
+            raise ValueError(f"{count} chosen tokens, room for {self.max_rows}")
+        if self.device.type != "cuda":       # no device: everything has happened already; keep a copy, since
+            return ChosenTokens(self.out[:count].clone(), None, count, None)     # the next step writes to ``out`` again
         landing = self._landing[self._turn]
         self._turn ^= 1
-        landing[:R].copy_(self.out[:R], non_blocking=True)
+        landing[:count].copy_(self.out[:count], non_blocking=True)
         ready = torch.cuda.Event()
         ready.record()
-        return ChosenTokens(self.out, landing, R, ready)
-
-    def sample(self, logits: torch.Tensor, temperatures, seeds, counters) -> list[int]:
-        """The same, waited for: token ids on the host."""
-        if logits.shape[0] == 0:
-            return []
-        return self.sample_async(logits, temperatures, seeds, counters).tolist()
+        return ChosenTokens(self.out, landing, count, ready)

@@ -287,3 +287,48 @@ def test_long_decoding_gpu(tiny_models):
     for i in (0, 1, 100, 250, 399):
         row = logits[len(prompt) - 1 + i]
         assert float(row.max() - row[out.output_ids[i]]) <= 1e-5
+
+
+def _tokens_chosen_in_the_step(m, device, backend, folder_or_config, weights, capture):
+    """Three requests decoded one token a step with sampling inputs handed to the step function: the tokens it
+    leaves in ``chosen_tokens`` must be what the sampling reference chooses from the logits it returns."""
+    from torch_backend import ref_sample
+    from mini_inference_engine_amd.engine.batch import StepRow
+    from mini_inference_engine_amd.engine.runner import ModelRunner
+    runner = ModelRunner(folder_or_config, weights=weights, dtype="float32", device=device, backend=backend, num_pages=16,
+                         max_rows=4, max_step_tokens=64)
+    if capture is not None:
+        runner.capture_decode_graphs((4,), sample=capture)
+    prompts = prompts_for(m, [7, 12, 3], seed=4)
+    caches = [runner.cache.open(i) for i in range(3)]
+    rows = []
+    for rc, p in zip(caches, prompts):
+        assert runner.cache.reserve(rc, 0, len(p))
+        rows.append(StepRow(rc, p, 0, [len(p) - 1]))
+    temps, seeds = [0.0, 0.9, 0.6], [0, 77, (5 << 32) + 9]
+    have = [len(p) for p in prompts]
+    logits = runner.forward_step(rows, sampling=(temps, seeds, [0, 0, 0]))          # portions: never captured
+    assert not runner.last_step_captured
+    for step in range(1, 5):
+        chosen = runner.chosen_tokens[:3].tolist()
+        expect = ref_sample(logits.cpu(), torch.tensor(temps), seeds, [step - 1] * 3).tolist()
+        assert chosen == expect, f"step {step}: the step chose {chosen}, the reference chooses {expect}"
+        rows = []
+        for i, rc in enumerate(caches):
+            assert runner.cache.reserve(rc, have[i], 1)
+            rows.append(StepRow(rc, [chosen[i]], have[i], [0]))
+            have[i] += 1
+        logits = runner.forward_step(rows, sampling=(temps, seeds, [step] * 3)).clone()
+        assert runner.last_step_captured == (capture is not None)
+
+
+def test_tokens_chosen_in_the_step_host(tiny_models):
+    m = tiny_models["A"]
+    _tokens_chosen_in_the_step(m, "cpu", TorchBackend(torch.float32), m["config"], m["weights"], None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("capture", [None, False, True], ids=["eager", "graphs", "graphs that sample"])
+def test_tokens_chosen_in_the_step_gpu(tiny_models, capture):
+    m = tiny_models["A"]
+    _tokens_chosen_in_the_step(m, "cuda", None, m["folder_f32"], None, capture)

@@ -119,7 +119,7 @@ def test_replay_through_captured_graphs(tiny_models, tmp_path, name, dtype, fami
     runner.capture_decode_graphs((1, 2, 4))
     replays = []
     run = runner.graphs.run
-    runner.graphs.run = lambda r, rows: (replays.append(len(rows)), run(r, rows))[1]
+    runner.graphs.run = lambda r, rows, sampling=None: (replays.append(len(rows)), run(r, rows, sampling))[1]
     run_replay(runner, steps, str(tmp_path))
     single = [len(s["entries"]) for s in steps if all(len(e["tokens"]) == 1 for e in s["entries"])]
     assert replays == single and len(single) >= 12, "steps of single tokens must all have been replayed from graphs"
