@@ -13,13 +13,19 @@ time K steps between device synchronisations.  Prints one JSON line:
   points    the same at batch 1 and 64, and at ``batch`` with contexts of 512; output and total tokens a second
             of the reference's mixed end-to-end workload (256 requests at once, prompts of 128..512 and outputs
             of 64..512 tokens; TinyLlama sizes only)
+            of 64..512 tokens; TinyLlama sizes only); prompts of 512, 4,096 and 8,192 tokens run in portions of at
+            most 2,048 (tokens a second over the whole prompt), and the last such portion of the longest alone
+            (2,048 new tokens behind 6,144 earlier ones)
   prefill   one 2,048-token prompt in one step: tokens a second, and flops / time / peak
   roofline  bytes a decode step must read (weights once + live cache) / time, against HBM peak
-Peaks: MI355X HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
+Peaks: MI355X HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.  Beside each fraction of a nominal
+peak stands ``frac_measured``: the same figure over what this GPU reaches in a plain microbenchmark run just
+before (a device-to-device copy of 1 GiB, bytes read + written; a library bfloat16 product of 8192^3).
 With --kernels no engine runs: the kernels a decode step and a prefill spend their time in are launched
 alone (captured in a graph, over rotating weight buffers so that nothing stays cached), and one JSON line
-lists for each its time, the bytes or flops it has to move or do and that over time over the peak
-(the reference's benchmarks/bench_kernels.py:1-79 does the same for its kernels, in GB/s).
+lists for each its time, the bytes or flops it has to move or do and that over time over the peak; then
+the reference's own grid (benchmarks/bench_kernels.py:30-72 there): add + RMSNorm at 1, 32, 256, 2,048 and 8,192
+rows of width 2,048, and decode attention at its eight (batch, context) points.
 The engine runs on one GPU; for --gpus > 1 one line says so and the exit code is 2.
 """
 from __future__ import annotations
@@ -79,6 +85,34 @@ def prefill_flops(cfg, tokens: int) -> float:
     return lin + att
 
 
+def measured_peaks() -> dict:
+    """What this GPU reaches in two plain microbenchmarks: a device-to-device copy of 1 GiB (bytes read +
+    written over time) and a library bfloat16 product of 8192 x 8192 x 8192 (flops over time)."""
+    import torch
+    def best(run, reps=5):
+        run()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            run()
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) * 1e-3)
+        return min(times)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    t_copy = best(lambda: dst.copy_(src))
+    del src, dst
+    a = torch.randn(8192, 8192, device="cuda").to(torch.bfloat16)
+    b = torch.randn(8192, 8192, device="cuda").to(torch.bfloat16)
+    t_mm = best(lambda: torch.mm(a, b.t()))
+    del a, b
+    torch.cuda.empty_cache()
+    return {"hbm_copy_GB_s": round(2 * (1 << 30) / t_copy / 1e9, 1), "bf16_gemm_PFLOP_s": round(2 * 8192.0 ** 3 / t_mm / 1e15, 3)}
+
+
 def prompts_of(n: int, length: int, vocab: int, seed: int):
     import torch
     g = torch.Generator().manual_seed(seed)
@@ -131,6 +165,43 @@ def measure_prefill(eng, tokens: int, seed: int):
         times.append(time.perf_counter() - t0)
         assert len(done) == 1 and done[0].num_computed == tokens, "the prompt did not run as one step"
     return min(times[1:])
+
+
+def measure_long_prefills(shape: str, layers, weights, dtype, lengths, block_size: int, seed: int):
+    """Prompts of ``lengths`` tokens under the step budget of 2,048 tokens: seconds for the whole prompt (in
+    portions of at most 2,048), and for the last portion alone.  The model is the same with positions enough for
+    the longest prompt (the layer sizes and weights do not depend on that)."""
+    import torch
+    from mini_inference_engine_amd import LLMEngine, SamplingParams
+    from mini_inference_engine_amd.config import EngineConfig, registry
+    longest = max(lengths)
+    over = {"max_position_embeddings": longest + 16}
+    if layers:
+        over["num_hidden_layers"] = layers
+    cfg = registry.shape_config(shape, **over)
+    ecfg = EngineConfig(block_size=block_size, max_num_seqs=2, max_num_batched_tokens=2048, max_model_len=longest + 16,
+                        num_blocks=-(-(longest + 16) // block_size) + 8, use_hip_graphs=False, run_ahead=False)
+    eng = LLMEngine(cfg, ecfg, dtype=dtype, verbose=False, weights=weights)
+    out = {}
+    for n in lengths:
+        best, best_last = None, None
+        for rep in range(4):
+            seq = eng.add_request(prompts_of(1, n, cfg.vocab_size, seed + rep)[0], SamplingParams(max_tokens=1, ignore_eos=True))
+            total, finished = 0.0, []
+            while not finished:
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                finished = eng.step()                    # a whole step: started, run and read (no running ahead here)
+                torch.cuda.synchronize()
+                last = time.perf_counter() - t0
+                total += last
+            assert finished == [seq] and seq.num_computed == n
+            if rep:                                      # the first run loads libraries and picks GEMM kernels
+                best, best_last = min(best or 1e9, total), min(best_last or 1e9, last)
+        out[n] = (best, best_last)
+    del eng
+    torch.cuda.empty_cache()
+    return out
 
 
 def measure_mixed(cfg, weights, dtype, requests: int, seed: int, use_graphs: bool):
@@ -277,8 +348,47 @@ def measure_kernels(cfg, args) -> int:
     w = weights(2 * inter, h)
     t = timed(lambda i: ops.linear(xt, w[i % copies]), copies)
     report(f"gate/up product (library), {T} rows", t, flops=2.0 * T * 2 * inter * h)
+    del w, qkv, xt, kc, vc
+    torch.cuda.empty_cache()
+    # ---- the reference's own grid (benchmarks/bench_kernels.py:30-72 there), at this shape's sizes
+    # add + RMSNorm: bytes as the reference counts them for its bfloat16 kernel (x, residual and y, and the residual
+    # written back: 4 x rows x width x 2) and what this kernel really moves (x bfloat16 in, the 32-bit stream in
+    # and out, y bfloat16 out)
+    norm_grid = []
+    for rows in (1, 32, 256, 2048, 8192):
+        xs = [torch.randn(rows, h, device=dev).to(torch.bfloat16) for _ in range(4)]
+        streams = [torch.randn(rows, h, device=dev) for _ in range(4)]
+        t = timed(lambda i: ops.add_rmsnorm(xs[i % 4], streams[i % 4], g_norm, cfg.rms_norm_eps), 8)
+        moved = rows * h * (2 + 4 + 4 + 2) + 2 * h
+        norm_grid.append({"rows": rows, "us": round(t * 1e6, 2), "GB_s": round(moved / t / 1e9, 1),
+                          "frac_hbm": round(moved / t / HBM_PEAK, 3),
+                          "GB_s_by_the_reference_count": round((4 * rows * h * 2 + 2 * h) / t / 1e9, 1)})
+    del xs, streams
+    attention_grid = []
+    for B, c in [(1, 512), (1, 2048), (8, 512), (8, 2048), (32, 512), (32, 1024), (64, 512), (128, 512)]:
+        per = -(-c // page)
+        kc = torch.randn(B * per + 1, Hkv, page, D, device=dev).to(torch.bfloat16)
+        vc = torch.randn(B * per + 1, Hkv, D, page, device=dev).to(torch.bfloat16)
+        bt = (torch.arange(B * per, device=dev, dtype=torch.int32) + 1).view(B, per).contiguous()
+        q = torch.randn(B, Hq * D, device=dev).to(torch.bfloat16)
+        st = SimpleNamespace(token_row=torch.arange(B, device=dev, dtype=torch.int32),
+                             positions=torch.full((B,), c - 1, device=dev, dtype=torch.int32), num_rows=B, max_context=c,
+                             num_tokens=B, num_decode_rows=B, max_row_tokens=1, row_start=None, row_position=None)
+        gr = SimpleNamespace(block_tables=bt, max_blocks=per)
+        t = timed(lambda i: ops.paged_attention(q, Hq, Hkv, D, kc, vc, gr, st, D ** -0.5, None), 8)
+        kv = 2 * B * c * Hkv * D * 2
+        attention_grid.append({"batch": B, "context": c, "us": round(t * 1e6, 2), "kv_GB_s": round(kv / t / 1e9, 1),
+                               "frac_hbm": round(kv / t / HBM_PEAK, 3)})
+        del kc, vc
+    peaks = measured_peaks()
+    for r in out + norm_grid + attention_grid:
+        if "GB_s" in r or "kv_GB_s" in r:
+            r["frac_measured"] = round(r.get("GB_s", r.get("kv_GB_s")) / peaks["hbm_copy_GB_s"], 3)
+        if "PFLOP_s" in r:
+            r["frac_measured"] = round(r["PFLOP_s"] / peaks["bf16_gemm_PFLOP_s"], 3)
     print(json.dumps({"metric": "kernel_times", "shape": SHAPE_NAMES[args.shape], "rows": M, "context": ctx,
-                      "peaks": {"hbm_GB_s": HBM_PEAK / 1e9, "bf16_PFLOP_s": FLOP_PEAK["bfloat16"] / 1e15}, "kernels": out}),
+                      "peaks": {"hbm_GB_s": HBM_PEAK / 1e9, "bf16_PFLOP_s": FLOP_PEAK["bfloat16"] / 1e15, "measured": peaks},
+                      "kernels": out, "add_rmsnorm": norm_grid, "decode_attention": attention_grid}),
           flush=True)
     return 0
 
@@ -316,6 +426,7 @@ def main() -> int:
         return measure_kernels(cfg, args)
     dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     elem = 2 if dtype == torch.bfloat16 else 4
+    peaks = measured_peaks()
     weights = random_tensors(cfg, args.seed, dtype, device="cuda")
     batches = sorted({args.batch} | (set() if args.no_points else {1, 64}))
     pages = max(batches) * (-(-args.context // args.block_size)) + 1 + 64
@@ -351,7 +462,8 @@ def main() -> int:
                    "page_size": args.block_size, "captured_steps": main_r["captured"], "parallelism": "single GPU",
                    "step": "LLMEngine.step: schedule + forward + sample, one step ahead of the token read-back"},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK, 4)},
+                     "frac": round(achieved / HBM_PEAK, 4), "peak_measured": peaks["hbm_copy_GB_s"],
+                     "frac_measured": round(achieved / 1e9 / peaks["hbm_copy_GB_s"], 4)},
     }
     if not args.no_points:
         line["points"] = {f"decode_b{b}": round(results[b]["tok_s"], 1) for b in (1, 64)}
@@ -361,9 +473,19 @@ def main() -> int:
         n = 2048 if args.context >= 2048 else args.context
         line["prefill"] = {"value": round(n / t, 1), "tokens": n, "ms": round(t * 1e3, 3),
                            "frac": round(prefill_flops(cfg, n) / t / FLOP_PEAK[args.dtype], 4)}
+        if dtype == torch.bfloat16:
+            line["prefill"]["peak_measured_PFLOP_s"] = peaks["bf16_gemm_PFLOP_s"]
+            line["prefill"]["frac_measured"] = round(prefill_flops(cfg, n) / t / 1e15 / peaks["bf16_gemm_PFLOP_s"], 4)
+        del eng
+        torch.cuda.empty_cache()
+        # longer and shorter prompts under the same 2,048-token step budget, and the last portion of the longest
+        lengths = [m for m in (512, 4096, 8192) if m != n]
+        for m, (whole, last) in measure_long_prefills(args.shape, args.layers, weights, dtype, lengths, args.block_size,
+                                                      args.seed + 200).items():
+            line["points"][f"prefill_{m}_tok_s"] = round(m / whole, 1)
+            if m == max(lengths) and m > 2048:
+                line["points"][f"prefill_2048_after_{m - 2048}_tok_s"] = round(2048 / last, 1)
         if args.shape == "tinyllama" and cfg.num_hidden_layers == full_layers and args.context >= 1024:
-            del eng
-            torch.cuda.empty_cache()
             mixed = measure_mixed(cfg, weights, dtype, 256, 0, not args.no_graphs)
             line["points"]["mixed_256_requests_output_tok_s"] = mixed["output_tok_s"]
             line["points"]["mixed_256_requests_total_tok_s"] = mixed["total_tok_s"]

@@ -29,6 +29,7 @@ class EngineConfig:
     activation_reserve_bytes: int = 768 * 2**20
     poison_freed_pages: bool = False        # debugging: fill returned pages with NaN
     run_ahead: bool = True                  # start a step before the host has read the tokens of the one before
+    trace_ranges: bool = False              # mark schedule / prepare / forward / sample of every step with profiler ranges
     cast_float32_weights: bool = False      # bfloat16 mode: round tensors the checkpoint stores in 32-bit to bfloat16
                                             # (the reference casts every tensor; by default they stay as stored)
 

@@ -73,7 +73,8 @@ class DecodeGraphs:
             sampling = ([0.0] * len(rows), [0] * len(rows), [0] * len(rows))     # nobody reads what is chosen
         step = runner.build(rows, pad_rows_to=bs, static_context=self.static_context, want_all=True, sampling=sampling)
         g, logits = self.graphs[bs]
-        g.replay()
+        with runner.ranges("forward"):       # (and "sample", when the graph chooses the tokens too)
+            g.replay()
         if not picked:
             return None, step
         if len(picked) == len(rows):

@@ -63,6 +63,8 @@ class LLMEngine:
             self.cache.on_release = self.runner.storage.poison_pages
         self.scheduler = Scheduler(self.cfg, self.cache)
         self.sampler = Sampler(self.runner.device, cfg.max_num_seqs, out=self.runner.chosen_tokens)
+        if cfg.trace_ranges and self.runner.device.type == "cuda":
+            self.runner.ranges.on = True
         self._in_flight = None             # the step whose tokens the host has not read yet
         self.stop_token_ids = frozenset(self.runner.model.spec.stop_token_ids)
         if verbose:
@@ -139,7 +141,8 @@ class LLMEngine:
         return finished
 
     def _start(self):
-        batch = self.scheduler.schedule()
+        with self.runner.ranges("schedule"):
+            batch = self.scheduler.schedule()
         if not batch:
             return None
         taken = self._in_flight.index_of if self._in_flight is not None else {}

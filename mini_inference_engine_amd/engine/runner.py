@@ -22,6 +22,21 @@ _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.
            torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
 
 
+class PhaseRanges:
+    """Named ranges around the phases of a step, for a profiler's timeline (rocprofv3 --marker-trace shows them;
+    the reference marks the same four phases with NVTX, inference_engine/engine.py:183-210).  Off by default:
+    ``ranges(name)`` is then an empty context."""
+
+    def __init__(self, on: bool = False):
+        self.on = bool(on)
+
+    def __call__(self, name: str):
+        if self.on:
+            return torch.cuda.nvtx.range(name)
+        import contextlib
+        return contextlib.nullcontext()
+
+
 def parse_dtype(d) -> torch.dtype:
     if d not in _DTYPES:
         raise ValueError(f"dtype {d!r}: choose bfloat16 or float32")
@@ -86,6 +101,7 @@ class ModelRunner:
         self.chosen_tokens = torch.zeros(max(1, max_rows), dtype=torch.int32, device=self.device)
         self.graphs = None                  # captured decode steps, once capture_decode_graphs was called
         self.last_step_captured = False
+        self.ranges = PhaseRanges(False)    # the entry point switches them on (EngineConfig.trace_ranges)
 
     # ------------------------------------------------------------------ steps
     def build(self, rows: list[StepRow], **kw):
@@ -95,7 +111,8 @@ class ModelRunner:
                                  f"{self.max_model_len}")
             if r.taken_from >= self.chosen_tokens.numel():
                 raise ValueError(f"a row takes its token from entry {r.taken_from} of {self.chosen_tokens.numel()}")
-        step = build_step(rows, self.arena, self.page_size, **kw)
+        with self.ranges("prepare"):
+            step = build_step(rows, self.arena, self.page_size, **kw)
         step.earlier_tokens = self.chosen_tokens
         return step
 
@@ -126,11 +143,13 @@ class ModelRunner:
                 return logits
         else:
             step = self.build(rows, sampling=sampling)
-            logits = self.model.forward(step)
+            with self.ranges("forward"):
+                logits = self.model.forward(step)
         if sampling is not None and logits is not None:
             n = logits.shape[0]
-            self.ops.sample(logits, step.sample_temps[:n], step.sample_seeds[:n], step.sample_counters[:n],
-                            out=self.chosen_tokens[:n])
+            with self.ranges("sample"):
+                self.ops.sample(logits, step.sample_temps[:n], step.sample_seeds[:n], step.sample_counters[:n],
+                                out=self.chosen_tokens[:n])
         return logits
 
     def after_step(self, rows: list[StepRow]) -> None:
