@@ -1,4 +1,4 @@
-// Matrix products of the bfloat16 path with 33 to 128 rows and a narrow weight (N up to a few thousand):
+// Matrix products of the bfloat16 path with 17 to 128 rows and a narrow weight (N up to a few thousand):
 // decode steps of many requests.  The few-row kernel (gemm_bf16.hip) gives every 16 weight rows a
 // workgroup that reads all of x, which at 64 rows is four times the weights' bytes; a library product
 // runs such a shape on a few dozen workgroups.  Here
@@ -30,7 +30,10 @@ union Frag {
 
 constexpr int MID_WAVES = 4;      // waves a workgroup = 16-row weight tiles a workgroup
 constexpr int MID_KC = 2;         // k-steps (of 32) a stage
-constexpr int MID_STAGES = 4;     // stages in the ring
+#ifndef MID_STAGES_OVERRIDE
+#define MID_STAGES_OVERRIDE 4
+#endif
+constexpr int MID_STAGES = MID_STAGES_OVERRIDE;     // stages in the ring
 constexpr int FRAG_BYTES = 1024;  // one operand fragment: 64 lanes x 16 bytes
 
 // wait until at most n vector memory loads of this wave are still on their way

@@ -154,7 +154,8 @@ class HipBackend(KernelBackend):
         return y
 
     # ---- few-row products of the bfloat16 path: one fused kernel each
-    SKINNY_MAX_ROWS = 32      # above this the split product or the library is faster than the fused kernel (measured at 24, 32, 48 rows)
+    SKINNY_MAX_ROWS = 16      # above this the split product or the library is faster than the fused kernel (decode steps of the
+                              # benchmark's sizes: 16 rows 1.24 against 1.28 ms; 24 rows 1.40 against 1.29; 32 rows 1.55 against 1.32)
     EPI_BF16, EPI_F32, EPI_ADD, EPI_SWIGLU = 0, 1, 2, 3
 
     def _skinny_ok(self, x, w, bias, rows=None) -> bool:
@@ -194,20 +195,19 @@ class HipBackend(KernelBackend):
                                                M, n_out, w.shape[1], *norm_args, self._stream()))
         return made
 
-    # ---- products of 33 to 128 rows on a narrow weight: split over K, partial results, one kernel that adds
+    # ---- products of 17 to 128 rows on a narrow weight: split over K, partial results, one kernel that adds
     # them up and does what follows the product
     MID_MAX_ROWS = 128
     MID_MAX_COLS = 4096        # wider weights have tiles enough for the library product without a split of K
     RED_BF16, RED_F32, RED_ADD, RED_ADD_NORM = 0, 1, 2, 3
 
     def _mid_ok(self, x, w, bias) -> bool:
-        """Whether the split product takes x w^T: 33 to 64 rows, or up to 128 where K is long (measured at the
-        benchmark's shapes: beyond 64 rows the library product with its separate epilogue kernel is as fast
-        unless K >= 4096)."""
+        """Whether the split product takes x w^T: more rows than the few-row kernel takes, up to 128 (measured at
+        the benchmark's shapes, decode steps of 80 / 96 / 128 rows with every narrow product here against the
+        library product and its separate epilogue kernel: 1.81 / 1.84 / 1.92 ms against 1.93 / 1.95 / 2.07)."""
         M = x.shape[0]
-        most = self.MID_MAX_ROWS if w.shape[1] >= 4096 else min(64, self.MID_MAX_ROWS)
         return (not self.true_fp32 and bias is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
-                and self.SKINNY_MAX_ROWS < M <= most and w.shape[0] <= self.MID_MAX_COLS
+                and self.SKINNY_MAX_ROWS < M <= self.MID_MAX_ROWS and w.shape[0] <= self.MID_MAX_COLS
                 and w.shape[0] % 4 == 0 and w.shape[1] % 8 == 0 and w.stride(0) % 8 == 0 and x.stride(0) % 8 == 0
                 and w.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0)
 
@@ -395,7 +395,7 @@ class HipBackend(KernelBackend):
 
     def _mid_rotary_kv_store(self, x, w_qkv, positions, cos, sin, Hq, Hkv, D, k_cache, v_cache, slot_mapping,
                              for_attention=False):
-        """The q/k/v projection of 33 to 128 rows: split product, then one kernel that adds the partial
+        """The q/k/v projection of 17 to 128 rows: split product, then one kernel that adds the partial
         results, rotates q and k and writes k and v to the cache.  Returns q [M, Hq * D] (for_attention: the
         partial results, for paged_attention to finish)."""
         self._on_device(x, w_qkv, positions, cos, sin, k_cache, v_cache, slot_mapping)

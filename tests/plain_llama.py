@@ -39,11 +39,12 @@ def rotate(x, cos, sin):
     return x * cos[:, None, :] + rot * sin[:, None, :]
 
 
-def causal_attention(q, k, v, scale, window=None):
+def causal_attention(q, k, v, scale, window=None, rounded=lambda t: t):
     """inference_engine/model.py:122-126,148-152: q [n, H, D], k, v [n, Hkv, D]; kv heads
     repeated H / Hkv times each (repeat_interleave), scores (q . k) scale, a query sees
     keys at or before it (and, with ``window``, at most window - 1 positions back: the
-    reference has no window), softmax over keys, times v."""
+    reference has no window), softmax over keys, times v.  ``rounded`` is applied to the
+    probabilities (see ``forward``'s ``act_round``)."""
     n, H, D = q.shape
     g = H // k.shape[1]
     ke = k.repeat_interleave(g, dim=1)
@@ -55,26 +56,26 @@ def causal_attention(q, k, v, scale, window=None):
     if window is not None:
         seen &= j > i - window
     s = s.masked_fill(~seen, float("-inf"))
-    p = torch.softmax(s, dim=-1)
+    p = rounded(torch.softmax(s, dim=-1))
     return torch.einsum("hij,jhd->ihd", p, ve)
 
 
-def swiglu(x, w_gate, w_up, w_down):
+def swiglu(x, w_gate, w_up, w_down, rounded=lambda t: t):
     """inference_engine/model.py:180-181: down(silu(gate(x)) * up(x)); silu(z) = z sigmoid(z)."""
     gate = x @ w_gate.T
     up = x @ w_up.T
-    return ((gate * torch.sigmoid(gate)) * up) @ w_down.T
+    return rounded((gate * torch.sigmoid(gate)) * up) @ w_down.T
 
 
-def attention_block(x, w, prefix, cfg, cos, sin):
+def attention_block(x, w, prefix, cfg, cos, sin, rounded=lambda t: t):
     """inference_engine/model.py:172-178: q,k,v projections, rotary on q and k, attention, o_proj."""
     n = x.shape[0]
     H, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     q = (x @ w[prefix + "q_proj.weight"].T).view(n, H, D)
     k = (x @ w[prefix + "k_proj.weight"].T).view(n, Hkv, D)
-    v = (x @ w[prefix + "v_proj.weight"].T).view(n, Hkv, D)
-    q, k = rotate(q, cos, sin), rotate(k, cos, sin)
-    o = causal_attention(q, k, v, 1.0 / math.sqrt(D))
+    v = rounded((x @ w[prefix + "v_proj.weight"].T).view(n, Hkv, D))
+    q, k = rounded(rotate(q, cos, sin)), rounded(rotate(k, cos, sin))
+    o = rounded(causal_attention(q, k, v, 1.0 / math.sqrt(D), rounded=rounded))
     return o.reshape(n, H * D) @ w[prefix + "o_proj.weight"].T
 
 
@@ -89,14 +90,22 @@ def normalise_config(cfg: dict) -> dict:
     return c
 
 
-def forward(cfg: dict, weights: dict, token_ids, dtype=torch.float64, position_offset: int = 0, rows=None):
+def forward(cfg: dict, weights: dict, token_ids, dtype=torch.float64, position_offset: int = 0, rows=None,
+            act_round=None):
     """Logits [n, vocab] of one whole sequence (inference_engine/model.py:161-185); with ``rows`` (a list of
     positions) only those rows of it, [len(rows), vocab], for sequences whose whole logits are too many.
     Residual wiring: stream = embed; stream += attention(norm(stream)); stream +=
     mlp(norm(stream)); logits = lm_head(norm(stream)).  ``position_offset`` shifts all
     positions (for the invariance test; the engine always starts at 0).  Runs where the
-    weights are (a model of real width is judged on the GPU, with torch's float64)."""
+    weights are (a model of real width is judged on the GPU, with torch's float64).
+
+    ``act_round`` (a dtype, e.g. torch.bfloat16): every activation that a reduced-precision pipeline has to
+    keep in that dtype is rounded to it once (normed inputs, q and k after the rotation, v, probabilities,
+    attention output, the feed-forward's activation), everything else stays in ``dtype``: the best any
+    implementation with activations of that dtype can do.  Its distance from the unrounded result is the noise
+    floor of the precision for this model and input; tests use it to tell a fault from rounding in deep models."""
     cfg = normalise_config(cfg)
+    rounded = (lambda t: t) if act_round is None else (lambda t: t.to(act_round).to(dtype))
     w = {k: v.to(dtype) for k, v in weights.items()}
     device = w["model.embed_tokens.weight"].device
     ids = torch.as_tensor(token_ids, dtype=torch.long, device=device)
@@ -107,14 +116,14 @@ def forward(cfg: dict, weights: dict, token_ids, dtype=torch.float64, position_o
     stream = w["model.embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
-        x = rms_norm(stream, w[p + "input_layernorm.weight"], eps)
-        stream = stream + attention_block(x, w, p + "self_attn.", cfg, cos, sin)
-        x = rms_norm(stream, w[p + "post_attention_layernorm.weight"], eps)
+        x = rounded(rms_norm(stream, w[p + "input_layernorm.weight"], eps))
+        stream = stream + attention_block(x, w, p + "self_attn.", cfg, cos, sin, rounded)
+        x = rounded(rms_norm(stream, w[p + "post_attention_layernorm.weight"], eps))
         stream = stream + swiglu(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
-                                 w[p + "mlp.down_proj.weight"])
+                                 w[p + "mlp.down_proj.weight"], rounded)
     if rows is not None:
         stream = stream[torch.as_tensor(rows, dtype=torch.long, device=device)]
-    x = rms_norm(stream, w["model.norm.weight"], eps)
+    x = rounded(rms_norm(stream, w["model.norm.weight"], eps))
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
     return x @ head.T
 

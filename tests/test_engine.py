@@ -230,7 +230,7 @@ def test_running_a_step_ahead_gpu(tiny_models, dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_many_requests_at_once_gpu(tiny_models, dtype):
-    """48 requests together: decode steps of 33 to 48 rows (beyond the few-row kernels), captured at batch
+    """48 requests together: decode steps of 33 to 48 rows (beyond the few-row kernels, which end at 16), captured at batch
     sizes 48 and 64, tokens handed from step to step on the device, greedy and sampled rows side by side."""
     m = tiny_models["B"]
     lengths = [1 + (7 * i) % 40 for i in range(48)]

@@ -6,10 +6,18 @@ there); here it is the logits that are compared, in float32 and in bfloat16:
   * one whole prompt of 300 tokens;
   * most of it in one step and the last 32 tokens one by one through the captured decode graph;
   * steps of 40 and of 64 single-token rows, launched kernel by kernel and through captured graphs
-    (the few-row kernels end at 32 rows; buckets 48 and 64).
+    (the few-row kernels end at 16 rows; buckets 48 and 64).
 
 The number of layers is LAYERS (the configuration has 22): what a layer does to the stream is the same in
 every layer, and the depth the engine's other tests reach is 3.
+
+Tolerances.  float32: 2e-5 of the request's logit scale, as everywhere.  bfloat16: 2e-2 of it, as everywhere, but
+never less than 1.5 times the noise floor of the precision: at this depth and width even an ideal pipeline, one
+that keeps everything in float64 and only rounds each stored activation to bfloat16 once
+(plain_llama.forward(act_round=torch.bfloat16)), ends 1.3e-2 to 1.6e-2 of the logit scale away from the unrounded
+result, its worst row among a few hundred; the engine, which rounds in a few more places (the library products'
+outputs), stands at 1.8e-2 to 2.0e-2 whatever the cut.  A bound of 2e-2 alone would sit inside the noise; the
+floor is measured for every request that is judged, so the bound follows the arithmetic and not the outcome.
 """
 import pytest
 import torch
@@ -55,6 +63,17 @@ def plain_logits(model, dtype, tokens):
     return plain_llama.forward(CFG, model[key], tokens, torch.float64)
 
 
+def bf16_tolerance(model, tokens, rows=None):
+    """max(BF16_TOL, 1.5 x the worst error of the ideal bfloat16 pipeline on these tokens), see the module's text."""
+    key = "bfloat16 widened"
+    if key not in model:
+        model[key] = {k: v.double() for k, v in model["bfloat16"].items()}
+    exact = plain_llama.forward(CFG, model[key], tokens, torch.float64, rows=rows)
+    ideal = plain_llama.forward(CFG, model[key], tokens, torch.float64, rows=rows, act_round=torch.bfloat16)
+    floor = float((ideal - exact).abs().max() / exact.abs().max())
+    return max(BF16_TOL, 1.5 * floor)
+
+
 def worst_error(got, expect, tol, what, scale=None):
     """got [n, vocab] float32 against expect [n, vocab] float64, in units of ``scale`` (the request's
     largest logit; by default the largest of ``expect``)."""
@@ -74,8 +93,8 @@ def prompt_tokens(n, seed):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_whole_prompt_then_tail_through_the_captured_graph(model, dtype):
     from mini_inference_engine_amd.engine.batch import StepRow
-    tol = F32_TOL if dtype == "float32" else BF16_TOL
     toks = prompt_tokens(PROMPT, 31)
+    tol = F32_TOL if dtype == "float32" else bf16_tolerance(model, toks)
     expect = plain_logits(model, dtype, toks)
     runner = make_runner(model, dtype, pages=2 * (PROMPT // 16 + 2) + 1, max_rows=4)
 
@@ -109,7 +128,6 @@ def test_decode_steps_of_40_and_64_rows(model, dtype, captured):
     """64 requests of 8 to 71 tokens.  All but their last two tokens go in as prompts (several a step);
     then one step of 40 single-token rows and one of 64."""
     from mini_inference_engine_amd.engine.batch import StepRow
-    tol = F32_TOL if dtype == "float32" else BF16_TOL
     lengths = [8 + (i * 37) % 64 for i in range(64)]
     requests = [prompt_tokens(n, 100 + i) for i, n in enumerate(lengths)]
     runner = make_runner(model, dtype, pages=sum(-(-n // 16) for n in lengths) + 1)
@@ -151,6 +169,7 @@ def test_decode_steps_of_40_and_64_rows(model, dtype, captured):
     worst = 0.0
     for i in range(64):
         expect = plain_logits(model, dtype, requests[i])
+        tol = F32_TOL if dtype == "float32" else bf16_tolerance(model, requests[i])
         for (j, p), row in got.items():
             if j == i:
                 worst = max(worst, worst_error(row[None], expect[p:p + 1], tol,
@@ -205,7 +224,7 @@ def test_captured_step_of_160_rows_replayed(model):
     worst = 0.0
     for i in range(0, n, 16):
         expect = plain_logits(model, dtype, requests[i])
-        worst = max(worst, worst_error(got[i][None], expect[fed[i] - 1:fed[i]], BF16_TOL, f"request {i}",
+        worst = max(worst, worst_error(got[i][None], expect[fed[i] - 1:fed[i]], bf16_tolerance(model, requests[i]), f"request {i}",
                                        scale=float(expect.abs().max())))
     print(f"160-row captured step: four replays equal the eager step; worst {worst:.2e} of the logit scale")
 
@@ -215,10 +234,10 @@ LONG = [640, 700, 610, 820, 660, 600]
 
 
 def compare_trace(model, dtype, prompts, got, what):
-    tol = F32_TOL if dtype == "float32" else BF16_TOL
     assert len(got) == sum(len(t) for t in prompts.values())
     worst = 0.0
     for rid, toks in prompts.items():
+        tol = F32_TOL if dtype == "float32" else bf16_tolerance(model, toks)
         expect = plain_logits(model, dtype, toks)
         rows = torch.stack([got[(rid, p)] for p in range(len(toks))])
         worst = max(worst, worst_error(rows, expect, tol, f"{what}: request {rid}"))
@@ -268,19 +287,18 @@ def test_mixed_steps_with_pages_used_again_at_full_width(model, dtype, captured)
           f"worst {worst:.2e} of the logit scale")
 
 
-SWEEP = (24, 33, 65, 96, 128, 129, 256)
+SWEEP = (16, 17, 33, 65, 96, 128, 129, 256)
 
 
 @pytest.mark.parametrize("captured", [False, True], ids=["eager", "graphs"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_decode_steps_from_24_to_256_rows(model, dtype, captured):
-    """One step of single-token rows at each of 24, 33, 65, 96, 128, 129 and 256 rows, launched kernel by kernel
-    and through captured graphs of exactly those sizes: the row counts at which the products change kernel
-    (few-row kernel to 32 rows, split product to 64, or to 128 for the down projection, the library beyond) and
-    at which the decode attention stops splitting contexts.  A sample of each step's rows against the plain
+def test_decode_steps_from_16_to_256_rows(model, dtype, captured):
+    """One step of single-token rows at each of 16, 17, 33, 65, 96, 128, 129 and 256 rows, launched kernel by
+    kernel and through captured graphs of exactly those sizes: the row counts at which the products change kernel
+    (few-row kernel to 16 rows, split product to 128 with 4 or 8 row tiles, the library beyond) and at which the
+    decode attention stops splitting contexts.  A sample of each step's rows against the plain
     implementation."""
     from mini_inference_engine_amd.engine.batch import StepRow
-    tol = F32_TOL if dtype == "float32" else BF16_TOL
     n_req, ahead = max(SWEEP), len(SWEEP)
     lengths = [10 + (i * 37) % 64 for i in range(n_req)]
     requests = [prompt_tokens(n, 2000 + i) for i, n in enumerate(lengths)]
@@ -318,8 +336,9 @@ def test_decode_steps_from_24_to_256_rows(model, dtype, captured):
     worst, expect_of = 0.0, {}
     for (n, i, p), row in got.items():
         if i not in expect_of:
-            expect_of[i] = plain_logits(model, dtype, requests[i])
-        e = expect_of[i]
+            expect_of[i] = (plain_logits(model, dtype, requests[i]),
+                            F32_TOL if dtype == "float32" else bf16_tolerance(model, requests[i]))
+        e, tol = expect_of[i]
         worst = max(worst, worst_error(row[None], e[p:p + 1], tol, f"{dtype}/{'graphs' if captured else 'eager'}: "
                                        f"step of {n} rows, row {i}, position {p}", scale=float(e.abs().max())))
     for rc in caches:

@@ -172,7 +172,7 @@ def test_skinny_linear(ops, shape):
     torch.testing.assert_close(stream, expect, atol=2e-3, rtol=2e-3)
 
 
-# --------------------------------------------------- products of 33 to 128 rows (bfloat16), split over K
+# --------------------------------------------------- products of 17 to 128 rows (bfloat16), split over K
 @pytest.fixture(scope="module")
 def engine_ops():
     """The backend with the engine's own thresholds between its three product paths."""
@@ -181,7 +181,7 @@ def engine_ops():
 
 
 MID_SHAPES = [(33, 2048, 2048), (64, 2048, 2560), (128, 5632, 2048), (50, 2008, 1000), (37, 256, 64), (100, 4104, 4096),
-              (65, 4096, 4), (40, 4096, 2048), (48, 8, 4)]
+              (65, 4096, 4), (40, 4096, 2048), (48, 8, 4), (17, 2048, 2048), (24, 520, 72), (128, 2048, 2560), (96, 264, 128)]
 
 
 @pytest.mark.parametrize("shape", MID_SHAPES)
@@ -199,9 +199,9 @@ def test_mid_linear(engine_ops, shape):
     assert y.dtype == torch.bfloat16
     torch.testing.assert_close(y.float(), exact.float(), atol=2e-2, rtol=1e-2)
     # a row's result does not depend on the rows beside it, nor on the number of row tiles
-    for a, b in ((0, 33), (M - 33, M), (0, min(M, 64))):
+    for a, b in ((0, 33), (max(0, M - 33), M), (0, min(M, 64))):
         assert torch.equal(o.linear(x[a:b].contiguous(), w, out_dtype=torch.float32), y32[a:b])
-    most = 128 if K >= 4096 else 64
+    most = 128
     big = torch.cat([x, x[:most - M]]) if M < most else x
     assert torch.equal(o.linear(big, w, out_dtype=torch.float32)[:M], y32)
     # residual add
@@ -239,15 +239,15 @@ def test_mid_linear_refuses_what_it_cannot_run(engine_ops):
 
 
 @pytest.mark.parametrize("geom", [(2, 1, 16), (3, 1, 32), (4, 2, 48), (32, 4, 64), (5, 5, 96), (8, 2, 128), (2, 1, 256)])
-@pytest.mark.parametrize("M", [40, 64])
+@pytest.mark.parametrize("M", [24, 40, 64, 128])
 def test_mid_projection_rotary_store(engine_ops, geom, M):
     """Split projection, then one kernel for sum + rotary + cache write, against the separate references
-    (K long enough for four splits at 40 rows, one split at 64)."""
+    (K long enough for four splits at 24, 40 and 128 rows, one split at 64)."""
     from mini_inference_engine_amd.parts.rope import rotary_tables
     Hq, Hkv, D = geom
     o = engine_ops
     torch.manual_seed(D + M)
-    K, page, pages = (1032 if M == 40 else 264), 16, 12
+    K, page, pages = (264 if M == 64 else 1032), 16, 12
     cos, sin = (t.to(DEV) for t in rotary_tables(10000.0, D, 300))
     x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
     w = (torch.randn((Hq + 2 * Hkv) * D, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
