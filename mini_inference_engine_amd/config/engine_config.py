@@ -29,6 +29,8 @@ class EngineConfig:
     activation_reserve_bytes: int = 768 * 2**20
     poison_freed_pages: bool = False        # debugging: fill returned pages with NaN
     run_ahead: bool = True                  # start a step before the host has read the tokens of the one before
+    tune_library_products: bool = True      # time the library's kernels once for the row counts that recur (graph batch
+                                            # sizes, the token budget) and keep the fastest; a few seconds at start-up
     trace_ranges: bool = False              # mark schedule / prepare / forward / sample of every step with profiler ranges
     cast_float32_weights: bool = False      # bfloat16 mode: round tensors the checkpoint stores in 32-bit to bfloat16
                                             # (the reference casts every tensor; by default they stay as stored)

@@ -54,7 +54,8 @@ class LLMEngine:
             num_pages=cfg.num_blocks, memory_fraction=cfg.kv_cache_memory_fraction,
             reserve_bytes=cfg.activation_reserve_bytes, max_step_tokens=cfg.max_num_batched_tokens,
             max_rows=cfg.max_num_seqs, max_model_len=cfg.max_model_len, num_state_slots=cfg.num_state_slots,
-            weights=weights, cast_float32_weights=cfg.cast_float32_weights)
+            weights=weights, cast_float32_weights=cfg.cast_float32_weights,
+            tune_library_products=cfg.tune_library_products)
         self.model_cfg = self.runner.model_cfg
         self.cfg.max_model_len = self.runner.max_model_len
         self.cache = self.runner.cache

@@ -47,7 +47,8 @@ class ModelRunner:
     def __init__(self, model, *, dtype=torch.bfloat16, device="cuda", backend=None, page_size: int = 16,
                  num_pages: int | None = None, memory_fraction: float = 0.85, reserve_bytes: int = 768 * 2**20,
                  max_step_tokens: int = 2048, max_rows: int = 256, max_model_len: int | None = None,
-                 num_state_slots: int | None = None, weights=None, cast_float32_weights: bool = False):
+                 num_state_slots: int | None = None, weights=None, cast_float32_weights: bool = False,
+                 tune_library_products: bool = False):
         """``model``: a folder with config.json and safetensors, or a ModelConfig together
         with ``weights`` (name -> tensor).  ``backend``: the kernels; by default the HIP
         library, which must load (there is no other product path)."""
@@ -66,6 +67,9 @@ class ModelRunner:
             from ..kernels.hip_backend import HipBackend
             backend = HipBackend(self.dtype, self.device)
         self.ops = backend
+        self.tune_library_products = bool(tune_library_products)
+        if self.tune_library_products:
+            backend.prefer_rows([max_step_tokens])    # a long prompt comes in portions of exactly the step's token budget
         self.model.use_backend(backend)
         self.load_report = load_weights(self.model, source, self.device, self.dtype, cast_float32=cast_float32_weights)
         self.model.prepare(self.device, self.dtype)
@@ -122,6 +126,8 @@ class ModelRunner:
         kernel (inference_engine/engine.py:76-120).  ``sample``: the captured step also chooses a token
         from every row's logits (for callers that pass ``sampling`` to ``forward_step``)."""
         from .graphs import DecodeGraphs
+        if self.tune_library_products:
+            self.ops.prefer_rows(batch_sizes)     # these row counts recur: the warm-up before each capture may choose kernels
         self.graphs = DecodeGraphs(self, batch_sizes, verbose=verbose, sample=sample)
 
     @torch.inference_mode()

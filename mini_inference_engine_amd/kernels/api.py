@@ -53,6 +53,10 @@ class KernelBackend:
     name = "?"
     act_dtype = None
 
+    def prefer_rows(self, counts) -> None:
+        """Row counts of steps that will recur (the batch sizes decode graphs are captured at, the token budget
+        of a step): a backend may spend time once, outside any capture, to choose its kernels for them."""
+
     def embedding(self, ids, table, taken_from=None, earlier_tokens=None):
         """stream[t, :] = float(table[ids[t], :]) -> [T, width] float32.  With ``taken_from`` (int32 [T]):
         where it is >= 0 the token is ``earlier_tokens[taken_from[t]]`` instead of ``ids[t]`` (a token the

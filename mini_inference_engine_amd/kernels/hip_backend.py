@@ -80,6 +80,9 @@ class HipBackend(KernelBackend):
             raise RuntimeError("no GPU visible to torch: the engine needs an MI355X (gfx950)")
         self._libs = {}
         self._zeros = None          # 256 zero bytes on the device, what masked loads of the mid-row product read
+        self._lt_workspace = None   # device memory the library's product kernels may use
+        self._lt_rows = set()       # row counts whose library products get their kernel chosen by timing (prefer_rows)
+        self._lt_tuned = set()      # (M, N, K, kind, leading dims) already chosen that way
         self.true_fp32 = act_dtype == torch.float32
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
 
@@ -100,6 +103,47 @@ class HipBackend(KernelBackend):
         for t in tensors:
             if t is not None and t.device.type != "cuda":
                 raise ValueError(f"tensor on {t.device}; the kernels take GPU tensors only")
+
+    # ---- library matrix products (many rows): hipBLASLt through csrc/lt_gemm.hip
+    LT_BF16, LT_F32, LT_ADD = 0, 1, 2
+    LT_WORKSPACE_BYTES = 128 << 20
+    LT_COLD_BYTES = 384 << 20       # overwritten before each timed launch of a finalist: more than the memory-side cache
+
+    def prefer_rows(self, counts) -> None:
+        self._lt_rows.update(int(c) for c in counts)
+
+    def _lt_ok(self, x, w) -> bool:
+        """Whether the engine's own call into the library takes x w^T (else torch's call does)."""
+        return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.stride(1) == 1 and w.stride(1) == 1
+                and w.shape[0] % 8 == 0 and w.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+                and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+    def _lt_product(self, x, w, kind, out):
+        """out (+)= x w^T by the library; out [M, N] contiguous, bfloat16 (LT_BF16) or float32."""
+        lib = self.lib("lt_gemm")
+        M, K = x.shape
+        N = w.shape[0]
+        if self._lt_workspace is None:
+            self._lt_workspace = torch.empty(self.LT_WORKSPACE_BYTES, dtype=torch.uint8, device=w.device)
+        ws = self._lt_workspace
+        if M in self._lt_rows:
+            key = (M, N, K, kind, x.stride(0), w.stride(0), out.stride(0))
+            if key not in self._lt_tuned and not torch.cuda.is_current_stream_capturing():
+                if not lib.mie_lt_is_tuned(x.stride(0), w.stride(0), out.stride(0), M, N, K, kind):
+                    # choose this shape's kernel by timing the library's suggestions, on a buffer that may be spoilt
+                    # (every kernel the library has for the shape; the finalists with the weights cold, as a step finds them)
+                    spoilt = out if kind != self.LT_ADD else torch.empty_like(out)
+                    cold = torch.empty(self.LT_COLD_BYTES, dtype=torch.uint8, device=w.device)
+                    best, first = c_float(0), c_float(0)
+                    library.check(lib, lib.mie_lt_tune(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(spoilt), spoilt.stride(0),
+                                                       M, N, K, kind, _ptr(ws), ws.numel(), 0, 5, _ptr(cold), cold.numel(),
+                                                       ctypes.byref(best), ctypes.byref(first), self._stream()))
+                    torch.cuda.current_stream().synchronize()
+                    del cold
+                self._lt_tuned.add(key)
+        library.check(lib, lib.mie_lt_gemm(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), M, N, K, kind,
+                                           _ptr(ws), ws.numel(), self._stream()))
+        return out
 
     # ----------------------------------------------------------------- ops
     def embedding(self, ids, table, taken_from=None, earlier_tokens=None):
@@ -292,15 +336,23 @@ class HipBackend(KernelBackend):
             # library matrix product, 32-bit accumulation, as the reference's F.linear.  What goes into the
             # float32 stream or out as logits leaves the product in float32: the sums are not rounded to
             # bfloat16 on their way there, whatever the number of rows.
+            own_call = bias is None and self._lt_ok(x, w)
             if bias is None and sink is not None:
                 # the product adds its float32 sums to the stream itself (C = C + A B in place): the stream is
                 # not read and written once more by a kernel of its own
-                torch.ops.aten.addmm.dtype_out(sink.stream, x, w.t(), torch.float32, out=sink.stream)
+                if own_call:
+                    self._lt_product(x, w, self.LT_ADD, sink.stream)
+                else:
+                    torch.ops.aten.addmm.dtype_out(sink.stream, x, w.t(), torch.float32, out=sink.stream)
                 if sink.norm_weight is None:
                     return None
                 return Normed(self, None, sink.stream, sink.norm_weight, sink.norm_eps)
             if bias is None and out_dtype == torch.float32:
+                if own_call:
+                    return self._lt_product(x, w, self.LT_F32, torch.empty((M, N), dtype=torch.float32, device=w.device))
                 return torch.mm(x, w.t(), out_dtype=torch.float32)
+            if own_call and out_dtype == torch.bfloat16:
+                return self._lt_product(x, w, self.LT_BF16, torch.empty((M, N), dtype=torch.bfloat16, device=w.device))
             y = torch.nn.functional.linear(x, w, None if bias is None else bias.to(torch.bfloat16))
             return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
         return self._gemm(x, w, bias, out_dtype)
@@ -358,7 +410,10 @@ class HipBackend(KernelBackend):
             M, K = x.shape
             page = self._check_rope_operands("linear_rotary_kv_store", M, K, w_qkv, positions, cos, sin, Hq, Hkv, D,
                                              k_cache, v_cache, slot_mapping)
-            sums = torch.mm(x, w_qkv.t(), out_dtype=torch.float32)
+            if self._lt_ok(x, w_qkv):
+                sums = self._lt_product(x, w_qkv, self.LT_F32, torch.empty((M, w_qkv.shape[0]), dtype=torch.float32, device=x.device))
+            else:
+                sums = torch.mm(x, w_qkv.t(), out_dtype=torch.float32)
             pending = ProjectionSums(self, sums[None], positions, cos, sin, slot_mapping, k_cache, v_cache, Hq, Hkv, D, page)
             return pending if for_attention else pending.finish()
         if not fused:

@@ -53,3 +53,10 @@ register_kernel_module("attention_bf16", {
 register_kernel_module("prefill_attention_bf16", {
     "mie_prefill_attention": [P, L, P, P, P, P, I, P, P, I, I, I, I, I, I, I, F, I, P],
 }, variants=_head_variants, flags=["-mllvm", "-amdgpu-mfma-vgpr-form"])
+# lt_gemm: host code only, the engine's own way into the library's matrix products (hipBLASLt) with the choice of
+# kernel per shape kept here.
+register_kernel_module("lt_gemm", {
+    "mie_lt_gemm": [P, L, P, L, P, L, I, I, I, I, P, L, P],
+    "mie_lt_is_tuned": [L, L, L, I, I, I, I],
+    "mie_lt_tune": [P, L, P, L, P, L, I, I, I, I, P, L, I, I, P, L, P, P, P],
+}, flags=["-L/opt/rocm/lib", "-lhipblaslt", "-Wl,-rpath,/opt/rocm/lib"])
