@@ -380,6 +380,26 @@ def measure_kernels(cfg, args) -> int:
         attention_grid.append({"batch": B, "context": c, "us": round(t * 1e6, 2), "kv_GB_s": round(kv / t / 1e9, 1),
                                "frac_hbm": round(kv / t / HBM_PEAK, 3)})
         del kc, vc
+    # ---- the library's products at M rows (the engine's own call, csrc/lt_gemm.hip): the kernel the library
+    # suggests first against the one kept after timing its kernels (what the engine does for row counts that recur)
+    library_grid = []
+    if M > 16:
+        for name, n_out, k, kind, odt in (("qkv, float32 sums", n_qkv, h, ops.LT_F32, torch.float32),
+                                          ("o, added into the stream", h, Hq * D, ops.LT_ADD, torch.float32),
+                                          ("gate/up, bfloat16", 2 * inter, h, ops.LT_BF16, torch.bfloat16),
+                                          ("down, added into the stream", h, inter, ops.LT_ADD, torch.float32)):
+            ws_ = weights(n_out, k)
+            xin = torch.randn(M, k, device=dev).to(torch.bfloat16)
+            dst = torch.zeros(M, n_out, device=dev, dtype=odt)
+            ops._lt_rows.discard(M)
+            first = timed(lambda i: ops._lt_product(xin, ws_[i % copies], kind, dst), copies)
+            ops.prefer_rows([M])
+            ops._lt_product(xin, ws_[0], kind, dst)              # times the library's kernels for this shape, keeps the fastest
+            tuned = timed(lambda i: ops._lt_product(xin, ws_[i % copies], kind, dst), copies)
+            library_grid.append({"product": name, "rows": M, "N": n_out, "K": k, "first_suggestion_us": round(first * 1e6, 2),
+                                 "kept_us": round(tuned * 1e6, 2), "GB_s": round(2 * n_out * k / tuned / 1e9, 1),
+                                 "PFLOP_s": round(2.0 * M * n_out * k / tuned / 1e15, 3)})
+            del ws_
     peaks = measured_peaks()
     for r in out + norm_grid + attention_grid:
         if "GB_s" in r or "kv_GB_s" in r:
@@ -388,7 +408,8 @@ def measure_kernels(cfg, args) -> int:
             r["frac_measured"] = round(r["PFLOP_s"] / peaks["bf16_gemm_PFLOP_s"], 3)
     print(json.dumps({"metric": "kernel_times", "shape": SHAPE_NAMES[args.shape], "rows": M, "context": ctx,
                       "peaks": {"hbm_GB_s": HBM_PEAK / 1e9, "bf16_PFLOP_s": FLOP_PEAK["bfloat16"] / 1e15, "measured": peaks},
-                      "kernels": out, "add_rmsnorm": norm_grid, "decode_attention": attention_grid}),
+                      "kernels": out, "add_rmsnorm": norm_grid, "decode_attention": attention_grid,
+                      "library_products": library_grid}),
           flush=True)
     return 0
 

@@ -153,9 +153,9 @@ MIE_EXPORT int mie_lt_is_tuned(long ldx, long ldw, long ldc, int M, int N, int K
 // Chooses this shape's kernel by timing, on ``stream`` (which must not be capturing).  candidates > 0: that many of
 // the library's suggestions; candidates = 0: every kernel the library has for these operand types that takes the
 // shape (hundreds).  First every candidate runs ``reps`` times back to back, operands warm; then the eight fastest
-// are timed one launch at a time with the weights cold, as a model's step finds them: before each launch ``cold``
-// (cold_bytes of device memory, more than the memory-side cache holds; may be null: then the warm times decide)
-// is overwritten.  C is written (and, for the adding kind, added to) over and over: give a buffer whose contents
+// and the library's first suggestion are timed one launch at a time with the weights cold, as a model's step finds
+// them: before each launch ``cold`` (cold_bytes of device memory, more than the memory-side cache holds; may be
+// null: then the warm times decide) is overwritten.  The first suggestion stays unless another is clearly faster.  C is written (and, for the adding kind, added to) over and over: give a buffer whose contents
 // do not matter.  best_us / first_us: the times of the kernel kept and of the library's first suggestion.
 MIE_EXPORT int mie_lt_tune(const void* X, long ldx, const void* W, long ldw, void* C, long ldc, int M, int N, int K, int kind,
                            void* workspace, long ws_bytes, int candidates, int reps, void* cold, long cold_bytes,
@@ -229,18 +229,27 @@ MIE_EXPORT int mie_lt_tune(const void* X, long ldx, const void* W, long ldw, voi
       std::vector<size_t> order;
       for (size_t f = 0; f < finalists; ++f) order.push_back(warm[f].second);
       if (!first_in && s[0].state == HIPBLAS_STATUS_SUCCESS) order.push_back(0);       // the library's own choice always competes
+      // the least of 2 x reps cold launches each (the least is what interference from outside cannot lower);
+      // another kernel replaces the library's own choice only if it is clearly faster: a microsecond and 3 %
+      float first_cold = -1.f;
       for (size_t i : order) {
-        float sum = 0.f;
+        float least = 1e30f;
         bool ok = true;
-        for (int r = 0; r < reps && ok; ++r) {
+        for (int r = 0; r < 2 * reps && ok; ++r) {
           const float us = time_of(i, 1, true);
           ok = us >= 0.f;
-          sum += us;
+          if (us < least) least = us;
         }
         if (!ok) continue;
-        const float us = sum / reps;
-        if (i == 0) first = us;
-        if (us < best) { best = us; keep = i; }
+        if (i == 0) first_cold = least;
+        if (least < best) { best = least; keep = i; }
+      }
+      if (first_cold > 0.f) {
+        first = first_cold;
+        if (keep != 0 && best > first_cold - (1.0f > 0.03f * first_cold ? 1.0f : 0.03f * first_cold)) {
+          keep = 0;
+          best = first_cold;
+        }
       }
     } else {
       best = warm[0].first;
