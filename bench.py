@@ -180,7 +180,7 @@ def measure_long_prefills(shape: str, layers, weights, dtype, lengths, block_siz
         over["num_hidden_layers"] = layers
     cfg = registry.shape_config(shape, **over)
     ecfg = EngineConfig(block_size=block_size, max_num_seqs=2, max_num_batched_tokens=2048, max_model_len=longest + 16,
-                        num_blocks=-(-(longest + 16) // block_size) + 8, use_hip_graphs=False, run_ahead=False)
+                        num_blocks=-(-(longest + 16) // block_size) + 8, graph_batch_sizes=(1,), run_ahead=False)
     eng = LLMEngine(cfg, ecfg, dtype=dtype, verbose=False, weights=weights)
     out = {}
     for n in lengths:

@@ -1,4 +1,5 @@
-"""Captured decode steps: one hipGraph per batch-size bucket.
+"""Captured steps: one hipGraph per batch-size bucket of single-token rows, and one for a prompt portion of
+exactly the step's token budget.
 
 A step of single-token rows is launch-bound when run kernel by kernel.  As in the
 reference (inference_engine/engine.py:76-120), the whole forward of such a step is
@@ -7,6 +8,12 @@ padded to its bucket with scratch rows that read and write page 0.  Everything a
 kernel needs that changes from step to step (token ids, positions, block tables,
 slots) is read from the arena on the device, so a replay needs only the arena's
 upload.  No memset node is recorded: buffers are cleared by kernels.
+
+A long prompt comes in portions of exactly the token budget of a step; such a step (one row, that many tokens,
+starting anywhere in its request, at most one position whose logits are wanted) has the same launches every time
+and is captured too (PortionGraph): launched kernel by kernel it costs the host about 3 ms, of which half a
+millisecond is not hidden behind the device when the engine was idle.  The reference captures single-token steps
+only.
 """
 from __future__ import annotations
 
@@ -80,3 +87,53 @@ class DecodeGraphs:
         if len(picked) == len(rows):
             return logits[:len(rows)], step
         return logits[torch.tensor(picked, device=logits.device)], step
+
+
+class _ScratchRequest:
+    """What a row needs of a request's cache, all of it the scratch page and the scratch slot: the row a step is
+    captured with."""
+
+    def __init__(self, num_groups: int, blocks: int):
+        self.tables = [[0] * blocks for _ in range(num_groups)]
+        self.state_slot = 0
+
+
+class PortionGraph:
+    """The captured step of one row of exactly ``tokens`` tokens with one row of logits."""
+
+    def __init__(self, runner, tokens: int, pool=None):
+        from .batch import StepRow
+        self.tokens = int(tokens)
+        self.static_context = runner.max_model_len
+        blocks = -(-self.tokens // runner.page_size)
+        scratch = _ScratchRequest(runner.arena.num_groups, blocks)
+        row = StepRow(scratch, [0] * self.tokens, 0, [self.tokens - 1])
+        step = runner.build([row], static_context=self.static_context)
+        runner.model.forward(step)                      # loads libraries, chooses the library's kernels, warms the allocator
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        collecting = gc.isenabled()
+        gc.disable()                                    # (as for the decode graphs: nothing is collected while the stream records)
+        try:
+            with torch.cuda.graph(self.graph, pool=pool):
+                self.logits = runner.model.forward(step)
+        finally:
+            if collecting:
+                gc.enable()
+        torch.cuda.synchronize()
+
+    def takes(self, rows) -> bool:
+        return (len(rows) == 1 and len(rows[0].tokens) == self.tokens and len(rows[0].want) <= 1
+                and rows[0].taken_from < 0)
+
+    def run(self, runner, rows, sampling=None):
+        """Logits [1, vocab] of the row's wanted position (None if it wants none), and the step as built."""
+        from .batch import StepRow
+        row = rows[0]
+        wanted = bool(len(row.want))
+        if not wanted:                                  # the graph computes one row of logits whatever happens: the last token's
+            row = StepRow(row.cache, row.tokens, row.start, [self.tokens - 1])
+        step = runner.build([row], static_context=self.static_context, sampling=sampling if wanted else None)
+        with runner.ranges("forward"):
+            self.graph.replay()
+        return (self.logits if wanted else None), step

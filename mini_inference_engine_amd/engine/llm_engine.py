@@ -84,6 +84,8 @@ class LLMEngine:
             self.tokenizer = AutoTokenizer.from_pretrained(model)
         if cfg.use_hip_graphs and self.runner.device.type == "cuda":
             self.runner.capture_decode_graphs(cfg.graph_batch_sizes, verbose=verbose, sample=True)
+            if cfg.enable_chunked_prefill and 2 <= cfg.max_num_batched_tokens <= self.runner.max_model_len:
+                self.runner.capture_portion_graph(cfg.max_num_batched_tokens)
         self.graphs = self.runner.graphs
         self.num_steps = 0
         self.num_graph_steps = 0

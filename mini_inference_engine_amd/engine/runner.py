@@ -104,6 +104,7 @@ class ModelRunner:
         # from here on the device (StepRow.taken_from) before the host has seen it.
         self.chosen_tokens = torch.zeros(max(1, max_rows), dtype=torch.int32, device=self.device)
         self.graphs = None                  # captured decode steps, once capture_decode_graphs was called
+        self.portion_graph = None           # the captured step of one full-budget prompt portion (capture_portion_graph)
         self.last_step_captured = False
         self.ranges = PhaseRanges(False)    # the entry point switches them on (EngineConfig.trace_ranges)
 
@@ -130,6 +131,19 @@ class ModelRunner:
             self.ops.prefer_rows(batch_sizes)     # these row counts recur: the warm-up before each capture may choose kernels
         self.graphs = DecodeGraphs(self, batch_sizes, verbose=verbose, sample=sample)
 
+    def capture_portion_graph(self, tokens: int | None = None) -> None:
+        """Capture the step that holds one prompt portion of exactly ``tokens`` tokens (default: the step's token
+        budget, what a long prompt is cut into); ``forward_step`` replays it for such steps."""
+        from .graphs import PortionGraph
+        tokens = int(tokens or self.arena.max_tokens)
+        if not 2 <= tokens <= min(self.arena.max_tokens, self.max_model_len):
+            raise ValueError(f"a captured portion of {tokens} tokens does not fit a step of {self.arena.max_tokens} "
+                             f"or a request of {self.max_model_len}")
+        if self.tune_library_products:
+            self.ops.prefer_rows([tokens])
+        pool = next(iter(self.graphs.graphs.values()))[0].pool() if self.graphs is not None and self.graphs.graphs else None
+        self.portion_graph = PortionGraph(self, tokens, pool=pool)
+
     @torch.inference_mode()
     def forward_step(self, rows: list[StepRow], sampling=None) -> torch.Tensor | None:
         """Logits [sum of wants, vocab] float32, ordered by row then by ``want``.
@@ -142,7 +156,10 @@ class ModelRunner:
         self.last_step_captured = False
         captured = (self.graphs is not None and self.graphs.fits(len(rows)) and all(len(r.tokens) == 1 for r in rows)
                     and (sampling is None or all(len(r.want) == 1 for r in rows)))
-        if captured:
+        if not captured and self.portion_graph is not None and self.portion_graph.takes(rows):
+            self.last_step_captured = True
+            logits, step = self.portion_graph.run(self, rows, sampling)
+        elif captured:
             self.last_step_captured = True
             logits, step = self.graphs.run(self, rows, sampling)
             if sampling is None or self.graphs.sample:

@@ -332,3 +332,49 @@ def test_tokens_chosen_in_the_step_host(tiny_models):
 def test_tokens_chosen_in_the_step_gpu(tiny_models, capture):
     m = tiny_models["A"]
     _tokens_chosen_in_the_step(m, "cuda", None, m["folder_f32"], None, capture)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_full_budget_portions_through_the_captured_graph(tiny_models, dtype):
+    """A prompt longer than the step's token budget comes in portions of exactly the budget; that step is
+    captured once and replayed (wherever in the request the portion starts, whether or not its logits are
+    wanted).  The same portions launched kernel by kernel by a second runner must give the same logits, bit for
+    bit in float32; then generation through the entry point, which reaches the graph by itself."""
+    from mini_inference_engine_amd.engine.batch import StepRow
+    from mini_inference_engine_amd.engine.runner import ModelRunner
+    m = tiny_models["B"]
+    folder = m["folder_f32"] if dtype == "float32" else m["folder_bf16"]
+    budget = 48
+    toks = prompts_for(m, [230], seed=9)[0]
+    runners = [ModelRunner(folder, dtype=dtype, device="cuda", num_pages=40, max_rows=4, max_step_tokens=budget)
+               for _ in range(2)]
+    runners[0].capture_portion_graph()
+    caches = [r.cache.open("a") for r in runners]
+    exact = plain_llama.forward(m["cfg"], m["weights"] if dtype == "float32" else m["weights_bf16"], toks)
+    start = 0
+    for n, want in ((budget, [budget - 1]), (7, [6]), (budget, []), (budget, [3]), (budget, [budget - 1]), (budget, [0, 1])):
+        outs = []
+        for r, rc in zip(runners, caches):
+            assert r.cache.reserve(rc, start, n)
+            out = r.forward_step([StepRow(rc, toks[start:start + n], start, want)])
+            outs.append(None if out is None else out.clone())
+        replayed = n == budget and len(want) <= 1
+        assert runners[0].last_step_captured == replayed and not runners[1].last_step_captured
+        if want:
+            if dtype == "float32":
+                assert torch.equal(outs[0], outs[1]), f"portion at {start}: the captured step differs from the launched one"
+            for o in outs:
+                err = (o.double().cpu() - exact[[start + w for w in want]]).abs().max() / exact.abs().max()
+                assert float(err) <= (2e-5 if dtype == "float32" else 2e-2), f"portion at {start}: {float(err):.2e}"
+        else:
+            assert outs[0] is None and outs[1] is None
+        start += n
+    # through the entry point: a prompt of 150 tokens under a budget of 48 is three captured portions and a rest
+    eng = engine(m, "cuda", dtype, num_blocks=40, max_num_seqs=4, max_num_batched_tokens=budget, graph_batch_sizes=(1, 2))
+    assert eng.runner.portion_graph is not None
+    prompts = prompts_for(m, [150], seed=10)
+    sp = SamplingParams(max_tokens=5, ignore_eos=True)
+    outs = eng.generate(prompts, sp)
+    assert eng.num_graph_steps >= 3 + 4, "three portions and the single-token steps after them must have been replayed"
+    check_outputs(m, prompts, outs, [sp], 1e-5 if dtype == "float32" else 2e-2, "weights" if dtype == "float32" else "weights_bf16")
