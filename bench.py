@@ -474,7 +474,9 @@ def main() -> int:
         "metric": "decode_tokens_per_second", "value": round(main_r["tok_s"], 1), "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(main_r["ms"], 4), "higher_is_better": True,
         "scaling": "weak",
-        "vs_baseline": round(main_r["tok_s"] / REFERENCE_B8_TOKENS_PER_S, 2) if args.batch == 8 and args.shape == "tinyllama" else None,
+        "vs_baseline": (round(main_r["tok_s"] / REFERENCE_B8_TOKENS_PER_S, 2)
+                        if args.batch == 8 and args.shape == "tinyllama" and cfg.num_hidden_layers == full_layers
+                        and dtype == torch.bfloat16 else None),
         "dtype": "bf16" if dtype == torch.bfloat16 else "fp32", "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
         "config": {"model": f"{SHAPE_NAMES[args.shape]} layer sizes (Llama)", "layers": cfg.num_hidden_layers, "layers_of_config": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
