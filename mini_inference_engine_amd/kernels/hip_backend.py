@@ -199,7 +199,8 @@ class HipBackend(KernelBackend):
 
     # ---- few-row products of the bfloat16 path: one fused kernel each
     SKINNY_MAX_ROWS = 16      # above this the split product or the library is faster than the fused kernel (decode steps of the
-                              # benchmark's sizes: 16 rows 1.24 against 1.28 ms; 24 rows 1.40 against 1.29; 32 rows 1.55 against 1.32)
+                              # benchmark's sizes: 16 rows 1.24 against 1.28 ms; 24 rows 1.40 against 1.29; 32 rows 1.55 against 1.32;
+                              # the same crossing at the layer sizes of Llama-2-7B and Llama-3-8B)
     EPI_BF16, EPI_F32, EPI_ADD, EPI_SWIGLU = 0, 1, 2, 3
 
     def _skinny_ok(self, x, w, bias, rows=None) -> bool:
@@ -242,7 +243,8 @@ class HipBackend(KernelBackend):
     # ---- products of 17 to 128 rows on a narrow weight: split over K, partial results, one kernel that adds
     # them up and does what follows the product
     MID_MAX_ROWS = 128
-    MID_MAX_COLS = 4096        # wider weights have tiles enough for the library product without a split of K
+    MID_MAX_COLS = 4096        # wider weights have tiles enough for the library product without a split of K (8192 measured
+                               # at hidden sizes of 4096: the same step times)
     RED_BF16, RED_F32, RED_ADD, RED_ADD_NORM = 0, 1, 2, 3
 
     def _mid_ok(self, x, w, bias) -> bool:
@@ -530,7 +532,9 @@ class HipBackend(KernelBackend):
         a workgroup; and with fewer workgroups where the contexts are short, because a workgroup then reads its
         whole context in less time than the merge kernel takes.  Measured at head size 64 (keys of 256 bytes a kv
         head): the unsplit kernel wins from 64 workgroups on at 512 keys, from 96 at 1,024, from 144 at 2,048:
-        about 32 + keys / 18."""
+        about 32 + keys / 18.  At head size 128 (8 and 32 kv heads, 1 to 16 rows, 512 to 8,192 keys) whole decode
+        steps with half the target, or unsplit at 512 keys, are within 3 % of this rule's, faster or slower by the
+        case: the rule holds there."""
         if window:
             context_bound = min(context_bound, window + 32)
         base = rows * Hkv * -(-(Hq // Hkv) // 16)
