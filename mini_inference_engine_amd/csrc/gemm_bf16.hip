@@ -1,15 +1,25 @@
-// Matrix products of the bfloat16 path with few rows (M <= 64: decode steps, the head on wanted rows),
+// Matrix products of the bfloat16 path with few rows (M <= 16: decode steps, the head on wanted rows),
 // where the weights are streamed once from HBM and everything else is noise: one kernel per product,
 // with what comes after it folded in, because at these sizes a launch costs as much as the work.
 //
 //   y[m, n] = sum_k x[m, k] W[n, k]          x [M, K], W [N, K] bfloat16 as stored in a checkpoint
 //
-// A workgroup of 4 or 8 waves owns 16 rows of W (one tile of C^T = W X^T); each wave streams one
-// contiguous quarter (eighth) of K in 32-wide steps, two groups of steps at a time;
-// v_mfma_f32_16x16x32_bf16 with A = 16 weight rows x 32 k (16 bytes a lane, straight from memory) and
-// B = 32 k x 16 batch rows; the waves' accumulators are summed through LDS in a fixed order.  A row's
-// result depends on nothing but that row, K, the weights and the number of waves (chosen from N alone):
-// it is bit-identical in any batch.
+// A workgroup of 4 waves owns 16 rows of W (one tile of C^T = W X^T); each wave streams one contiguous
+// quarter of K in 32-wide steps; v_mfma_f32_16x16x32_bf16 with A = 16 weight rows x 32 k and B = 32 k x 16
+// batch rows; the waves' accumulators are summed through LDS in a fixed order.  A row's result depends on
+// nothing but that row, K and the weights: it is bit-identical in any batch.
+//
+// How the operands reach the matrix instruction.  The instruction wants lane 16 b + r to hold k-block b (8
+// values, 16 bytes) of row r.  Loaded in that order, a quarter wave (16 lanes) touches 16 cache lines for 16
+// bytes each, and the address unit, which looks lines up one at a time, is then what bounds the kernel: the x
+// loads alone (all of them hits) cost a seventh to a third of its time, and the weights stream at 4.2 to
+// 4.7 TB/s where a plain read of the same bytes runs at 5.4 to 5.8.  So the loads are issued in the order lane
+// 4 r + b (a quarter wave reads 64 contiguous bytes of 4 rows) and write the wave's own piece of the LDS
+// directly (no registers, nothing the compiler waits for): a ring of slots of two k-steps, all but one on their
+// way while that one is multiplied.  Within a row the four blocks are permuted (block b at 16-byte slot
+// 4 r + (b ^ (r / 4) % 4)), so that the fragment reads (lane 16 b + r) are spread over all banks.  No barrier
+// in the loop: a wave reads only what it brought in itself.  (The same order with nontemporal loads reads a
+// fifth faster still when nothing else is loaded, but slower beside the x loads: measured, not used.)
 //
 // Epilogues: STORE (bfloat16 or float32 y), ADD (r[m, n] += y, the residual add of the 32-bit stream),
 //   SWIGLU (W holds gate rows then up rows; a tile is 8 gate rows and the matching 8 up rows, and the
@@ -19,22 +29,42 @@
 // converted the 32-bit stream inside every workgroup was measured and dropped: redoing the conversion of
 // all of x per workgroup cost more than a separate norm kernel.)
 #include "common.hpp"
+#include <mutex>
+#include <set>
+#include <stdlib.h>
+#include <utility>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-union Frag {
-  bf16x8 v;
-  uint4 q;
-  uint32_t w[4];
-};
+// what a k-step beyond a wave's range or beyond K loads instead of weights, so that every load is unconditional
+__device__ __align__(64) const uint32_t mie_zero_words[16] = {0};
 
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-  uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
-  ua += 0x7FFFu + ((ua >> 16) & 1u);
-  ub += 0x7FFFu + ((ub >> 16) & 1u);
-  return (ua >> 16) | (ub & 0xFFFF0000u);
-}
+// wait until at most n vector memory loads of this wave are still on their way
+#define SG_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+constexpr int SG_WAVES = 4;       // waves a workgroup
+constexpr int SG_THREADS = SG_WAVES * 64;
+constexpr int RING_U = 2;         // k-steps a slot of a wave's ring
+
+// The fragments of a slot (U k-steps: weight fragment, x fragment, 1 KB each) out of the LDS, read and waited for
+// in one piece of assembly: the compiler knows nothing of the loads that write the LDS, so a read it could see
+// would make it wait for every load on its way, and it must never see a register whose value is still to arrive.
+typedef uint32_t sg_u32x4 __attribute__((ext_vector_type(4)));
+template <int U> struct RingRead;
+template <> struct RingRead<2> {
+  static __device__ __forceinline__ void run(uint32_t at, sg_u32x4 (&f)[4]) {
+    asm volatile(
+      "ds_read_b128 %0, %4\n\t"
+      "ds_read_b128 %1, %4 offset:1024\n\t"
+      "ds_read_b128 %2, %4 offset:2048\n\t"
+      "ds_read_b128 %3, %4 offset:3072\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3])
+      : "v"(at)
+      : "memory");
+  }
+};
 
 enum { EPI_STORE_BF16 = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3, EPI_ROPE = 4 };
 
@@ -91,17 +121,17 @@ __device__ __forceinline__ long tile_column(int tile, int c, int N, int up_offse
   return n;
 }
 
-template <int MT, int EPI, int WAVES, bool NF>
-__global__ void __launch_bounds__(WAVES * 64)
+template <int EPI, bool NF, int SLOTS>
+__global__ void __launch_bounds__(SG_THREADS)
 skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict__ W, long ldw, void* __restrict__ outv,
                    long ldo, int M, int N, int K, int up_offset, RopeArgs rope, NormArgs nf) {
-  // k-steps per group of loads (two groups are in flight per wave)
-  constexpr int U = MT == 1 ? 4 : 2;
-  constexpr int SG_WAVES = WAVES;
-  constexpr int SG_THREADS = WAVES * 64;
-  constexpr int PER = (MT * 256 + SG_THREADS - 1) / SG_THREADS;   // results (m, n) a thread owns after the reduction
-  __shared__ float s_acc[SG_WAVES][MT][256];
-  __shared__ float s_rstd[MT * 16];
+  constexpr int SLOT_BYTES = RING_U * 2 * 1024;            // a k-step: the weight fragment, then the x fragment, 1 KB each
+  constexpr int WAVE_BYTES = SLOTS * SLOT_BYTES;
+  constexpr int L = RING_U * 2;                            // loads a slot
+  static_assert((SLOTS - 1) * L <= 63, "more loads in flight than the counter holds");
+  extern __shared__ __align__(16) char ring_lds[];         // WAVE_BYTES a wave
+  __shared__ float s_acc[SG_WAVES][256];
+  __shared__ float s_rstd[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kb = lane >> 4;
   const int tile = blockIdx.x;
@@ -110,233 +140,195 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
   const int ks0 = wave * per_wave;
   const int ks1 = ks0 + per_wave < ksteps ? ks0 + per_wave : ksteps;
 
-  // What the epilogue reads beside the product is asked for first, so that it has arrived long before it is used.
-  float e_old[PER], e_cos[PER], e_sin[PER];
-  uint32_t e_g[PER];                       // raw bits of the next norm's weight (converted where it is used)
-  int e_slot[PER], e_pos[PER];
-  bool e_live[PER];
-  long e_n[PER];
-#pragma unroll
-  for (int j = 0; j < PER; ++j) {
-    const int e = threadIdx.x + j * SG_THREADS;
-    const int m = e >> 4;
-    bool ok;
-    e_n[j] = tile_column<EPI>(tile, e & 15, N, up_offset, rope.D, ok);
-    e_live[j] = e < MT * 256 && m < M && ok;
-    // every load below is unconditional, from an address clamped into the operand
-    const int mc = e_live[j] ? m : 0;
-    const long nc = e_live[j] ? e_n[j] : 0;
-    e_old[j] = e_cos[j] = e_sin[j] = 0.f;
-    e_g[j] = 0u;
-    e_slot[j] = e_pos[j] = 0;
-    if (EPI == EPI_ADD) {
-      e_old[j] = ((const float*)outv)[(size_t)mc * ldo + nc];
-      if (NF) e_g[j] = nf.g_f32 ? ((const uint32_t*)nf.g)[nc] : (uint32_t)((const uint16_t*)nf.g)[nc];
-    }
-    if (EPI == EPI_ROPE) {
-      e_pos[j] = rope.positions[mc];
-      e_slot[j] = rope.slots[mc];
-    }
+  // What this lane brings in: row lrow (of the weight tile; of x), k-block lkb of every k-step.  And the one
+  // result this thread owns after the waves are summed: x row m, column c of the tile.  The gather of x's
+  // rows, if there is one, is the first thing asked for: addresses depend on it.
+  const int lrow = lane >> 2, lkb = (lane & 3) ^ ((lrow >> 2) & 3);
+  const int m = threadIdx.x >> 4, c = threadIdx.x & 15;
+  const bool gather = NF && EPI != EPI_ADD && nf.rows;
+  const int lsrc = lrow < M ? (gather ? nf.rows[lrow] : lrow) : 0;
+  const int msrc = m < M ? (gather ? nf.rows[m] : m) : 0;
+
+  // What the epilogue reads beside the product is asked for next, so that it has arrived long before it is
+  // used and is older than every load of the ring (the counter of loads on their way runs in issue order).
+  // Every load is unconditional, from an address clamped into the operand.
+  bool ok;
+  const long n = tile_column<EPI>(tile, c, N, up_offset, rope.D, ok);
+  const bool live = m < M && ok;
+  const int mc = live ? m : 0;
+  const long nc = live ? n : 0;
+  float e_old = 0.f, e_cos = 0.f, e_sin = 0.f;
+  uint32_t e_g = 0u;                       // raw bits of the next norm's weight (converted where it is used)
+  int e_slot = 0, e_pos = 0;
+  if (EPI == EPI_ADD) {
+    e_old = ((const float*)outv)[(size_t)mc * ldo + nc];
+    if (NF) e_g = nf.g_f32 ? ((const uint32_t*)nf.g)[nc] : (uint32_t)((const uint16_t*)nf.g)[nc];
   }
-  // Fused norm, consuming side: the partial sums of squares likewise.  16 lanes a row, lane sub takes
-  // the tiles 4 (sub + 16 i) .. + 3: the first SSP fours now, the rest (widths above 4096) after the loop.
+  if (EPI == EPI_ROPE) {
+    e_pos = rope.positions[mc];
+    e_slot = rope.slots[mc];
+  }
+  // Fused norm, consuming side: the partial sums of squares likewise.  16 lanes a row, lane c takes the
+  // tiles 4 (c + 16 i) .. + 3: the first SSP fours now, the rest (widths above 4096) after the loop.
   constexpr int SSP = 4;
-  float4 ssp[PER][SSP];
+  float4 ssp[SSP];
   const int ss_ld = (nf.ss_tiles + 3) & ~3;
   if (NF && EPI != EPI_ADD) {
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int e = threadIdx.x + j * SG_THREADS;
-      const int mm = (e >> 4) < MT * 16 ? (e >> 4) : 0, sub = e & 15;
-      const int src = mm < M ? (nf.rows ? nf.rows[mm] : mm) : 0;
-#pragma unroll
-      for (int i = 0; i < SSP; ++i) {
-        const int t = 4 * (sub + 16 * i);
-        ssp[j][i] = *reinterpret_cast<const float4*>(nf.ss_in + (size_t)src * ss_ld + (t < ss_ld ? t : 0));
-      }
+    for (int i = 0; i < SSP; ++i) {
+      const int t = 4 * (c + 16 * i);
+      ssp[i] = *reinterpret_cast<const float4*>(nf.ss_in + (size_t)msrc * ss_ld + (t < ss_ld ? t : 0));
     }
   }
 
-  // weight row of this lane (clamped for the address; a row that does not exist is never stored)
-  bool wok;
-  const long wr = tile_column<EPI>(tile, col, N, up_offset, rope.D, wok);
-  const bf16* wrow = W + (size_t)(wok ? wr : 0) * ldw;
-  // batch rows of this lane; lanes of rows beyond M read row 0 along with the lanes that own it
-  const bf16* xrow[MT];
+  // The ring.  Slots beyond the wave's range load zeros only, so that it is always filled and drained the
+  // same way.
+  bool lok;
+  const long lwr = tile_column<EPI>(tile, lrow, N, up_offset, rope.D, lok);
+  const bf16* wsrc = W + (size_t)(lok ? lwr : 0) * ldw + lkb * 8;   // a row that does not exist is never stored
+  const bf16* xsrc = X + (size_t)lsrc * ldx + lkb * 8;              // rows beyond M read row 0 along with the lanes that own it
+  const bf16* zero_lane = reinterpret_cast<const bf16*>(mie_zero_words) + lkb * 8;   // per lane, so that choosing it is a select
+  char* mine = ring_lds + wave * WAVE_BYTES;
+  auto issue = [&](int s) {
+    char* base = mine + (s % SLOTS) * SLOT_BYTES;
+    const int ks = ks0 + s * RING_U;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + col;
-    const int src = m < M ? (NF && EPI != EPI_ADD && nf.rows ? nf.rows[m] : m) : 0;
-    xrow[mt] = X + (size_t)src * ldx;
-  }
-
-  f32x4 acc[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  // One group = U k-steps.  load_group only issues loads (raw values into registers) and notes which
-  // steps count; the zeroing of steps that do not count happens in multiply(), so no load is waited
-  // for where it is issued.  Every load is unconditional, from an address clamped into the operand
-  // (k 0 for steps beyond this wave's range).
-  struct Group {
-    uint4 a[U];
-    uint4 b[U][MT];
-    bool ok[U];
-  };
-  auto load_group = [&](Group& G, int ks) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int k = (ks + u) * 32 + kb * 8;
-      const bool kok = ks + u < ks1 && k < K;
-      const int kc = kok ? k : 0;
-      G.ok[u] = kok;
-      G.a[u] = *reinterpret_cast<const uint4*>(wrow + kc);
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) G.b[u][mt] = *reinterpret_cast<const uint4*>(xrow[mt] + kc);
+    for (int u = 0; u < RING_U; ++u) {
+      const bool kok = ks + u < ks1 && (ks + u) * 32 + lkb * 8 < K;
+      const bf16* a = kok ? wsrc + (size_t)(ks + u) * 32 : zero_lane;
+      const bf16* b = kok ? xsrc + (size_t)(ks + u) * 32 : zero_lane;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)a,
+                                       (__attribute__((address_space(3))) void*)(base + (2 * u) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)b,
+                                       (__attribute__((address_space(3))) void*)(base + (2 * u + 1) * 1024), 16, 0, 0);
     }
   };
-  auto multiply = [&](Group& G) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const bool kok = G.ok[u];
-      Frag a, b[MT];
-      const uint4 w = G.a[u];
-      a.q = make_uint4(kok ? w.x : 0u, kok ? w.y : 0u, kok ? w.z : 0u, kok ? w.w : 0u);   // a step that does not count
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) b[mt].q = G.b[u][mt];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[mt].v, acc[mt], 0, 0, 0);
-    }
-  };
-
-  Group g0, g1;
-  load_group(g0, ks0);
+  const int rounds = ks1 > ks0 ? (ks1 - ks0 + RING_U - 1) / RING_U : 0;
+  // this lane's piece of a fragment: row col, block kb
+  const uint32_t at0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)mine + (col * 4 + (kb ^ ((col >> 2) & 3))) * 16;
+  for (int s = 0; s < SLOTS - 1; ++s) issue(s);
   if (EPI == EPI_ROPE) {
-    // the angles, once the positions are here (they were asked for before the first group)
+    // the angles, once the positions are here (asked for before the ring: waiting for them does not wait for it)
     const int half = rope.D >> 1;
+    const int per_head = rope.D >> 4;
+    const int jd = (tile % per_head) * 8 + (c & 7);
+    e_cos = rope.cos_t[(size_t)e_pos * half + jd];       // position 0 for the rows that do not count
+    e_sin = rope.sin_t[(size_t)e_pos * half + jd];
+  }
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int it = 0; it < rounds; ++it) {
+    issue(it + SLOTS - 1);                         // into the slot that was read a round ago
+    SG_VMCNT((SLOTS - 1) * L);                     // slot `it` has landed (anything asked for in between only makes this wait for more)
+    sg_u32x4 f[2 * RING_U];
+    RingRead<RING_U>::run(at0 + (it % SLOTS) * SLOT_BYTES, f);
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int e = threadIdx.x + j * SG_THREADS;
-      const int per_head = rope.D >> 4;
-      const int jd = (tile % per_head) * 8 + (e & 7);
-      e_cos[j] = rope.cos_t[(size_t)e_pos[j] * half + jd];       // position 0 for the rows that do not count
-      e_sin[j] = rope.sin_t[(size_t)e_pos[j] * half + jd];
-    }
+    for (int u = 0; u < RING_U; ++u)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, f[2 * u]), __builtin_bit_cast(bf16x8, f[2 * u + 1]),
+                                                    acc, 0, 0, 0);
   }
-  for (int ks = ks0; ks < ks1; ks += 2 * U) {
-    load_group(g1, ks + U);          // in flight while group 0 is multiplied
-    multiply(g0);
-    load_group(g0, ks + 2 * U);
-    multiply(g1);
-  }
+  SG_VMCNT(0);                                     // nothing of this wave may still be writing the LDS when it ends
 
   if (NF && EPI != EPI_ADD) {
     // 1 / sqrt(mean of squares + eps) of every row, summed in a fixed order
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int e = threadIdx.x + j * SG_THREADS;
-      const int mm = (e >> 4) < MT * 16 ? (e >> 4) : 0, sub = e & 15;
-      float sum = 0.f;
-#pragma unroll
-      for (int i = 0; i < SSP; ++i) {
-        const int t = 4 * (sub + 16 * i);
-        sum += (t < nf.ss_tiles ? ssp[j][i].x : 0.f) + (t + 1 < nf.ss_tiles ? ssp[j][i].y : 0.f) +
-               (t + 2 < nf.ss_tiles ? ssp[j][i].z : 0.f) + (t + 3 < nf.ss_tiles ? ssp[j][i].w : 0.f);
-      }
-      if (nf.ss_tiles > 64 * SSP) {
-        const int src = mm < M ? (nf.rows ? nf.rows[mm] : mm) : 0;
-        for (int t = 64 * SSP + sub; t < nf.ss_tiles; t += 16) sum += nf.ss_in[(size_t)src * ss_ld + t];
-      }
-      sum += __shfl_xor(sum, 1, 64);
-      sum += __shfl_xor(sum, 2, 64);
-      sum += __shfl_xor(sum, 4, 64);
-      sum += __shfl_xor(sum, 8, 64);
-      if (sub == 0 && e < MT * 256) s_rstd[mm] = 1.0f / sqrtf(sum * nf.inv_width + nf.eps);
-    }
-  }
-
-  // sum the waves, each thread owning elements (m, c) = (e / 16, e % 16)
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) s_acc[wave][mt][lane * 4 + i] = acc[mt][i];
-  __syncthreads();
-  float v[PER];
-#pragma unroll
-  for (int j = 0; j < PER; ++j) {
-    const int e = threadIdx.x + j * SG_THREADS;
     float sum = 0.f;
-    if (e < MT * 256) {
-      const int mm = e >> 4, nn = e & 15;
-      const int src = (((nn >> 2) << 4) + (mm & 15)) * 4 + (nn & 3);
 #pragma unroll
-      for (int w = 0; w < SG_WAVES; ++w) sum += s_acc[w][mm >> 4][src];
+    for (int i = 0; i < SSP; ++i) {
+      const int t = 4 * (c + 16 * i);
+      sum += (t < nf.ss_tiles ? ssp[i].x : 0.f) + (t + 1 < nf.ss_tiles ? ssp[i].y : 0.f) +
+             (t + 2 < nf.ss_tiles ? ssp[i].z : 0.f) + (t + 3 < nf.ss_tiles ? ssp[i].w : 0.f);
     }
-    v[j] = sum;
+    if (nf.ss_tiles > 64 * SSP)
+      for (int t = 64 * SSP + c; t < nf.ss_tiles; t += 16) sum += nf.ss_in[(size_t)msrc * ss_ld + t];
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    sum += __shfl_xor(sum, 4, 64);
+    sum += __shfl_xor(sum, 8, 64);
+    if (c == 0) s_rstd[m] = 1.0f / sqrtf(sum * nf.inv_width + nf.eps);
   }
 
+  // sum the waves: acc[i] of lane (col, kb) is weight row 4 kb + i (column of the tile), x row col
 #pragma unroll
-  for (int j = 0; j < PER; ++j) {
-    const int e = threadIdx.x + j * SG_THREADS;
-    const int m = e >> 4, c = e & 15;
-    const bool live = e_live[j];
-    const long n = e_n[j];
-    if (EPI == EPI_ADD) {
-      const float r = e_old[j] + v[j];
-      if (live) ((float*)outv)[(size_t)m * ldo + n] = r;
-      if (NF) {
-        const float g = nf.g_f32 ? __uint_as_float(e_g[j]) : __uint_as_float(e_g[j] << 16);
-        if (live) nf.x_next[(size_t)m * nf.ldx_next + n] = __float2bfloat16(r * g);
-        float q = live ? r * r : 0.f;          // the 16 lanes of a row: sum of squares over this tile's columns
-        q += __shfl_xor(q, 1, 64);
-        q += __shfl_xor(q, 2, 64);
-        q += __shfl_xor(q, 4, 64);
-        q += __shfl_xor(q, 8, 64);
-        if (c == 0 && e < MT * 256 && m < M) nf.ss_out[(size_t)m * ((gridDim.x + 3) & ~3) + tile] = q;
-      }
-      continue;
+  for (int i = 0; i < 4; ++i) s_acc[wave][lane * 4 + i] = acc[i];
+  __syncthreads();
+  float v = 0.f;
+  {
+    const int src = (((c >> 2) << 4) + m) * 4 + (c & 3);
+#pragma unroll
+    for (int w = 0; w < SG_WAVES; ++w) v += s_acc[w][src];
+  }
+
+  if (EPI == EPI_ADD) {
+    const float r = e_old + v;
+    if (live) ((float*)outv)[(size_t)m * ldo + n] = r;
+    if (NF) {
+      const float g = nf.g_f32 ? __uint_as_float(e_g) : __uint_as_float(e_g << 16);
+      if (live) nf.x_next[(size_t)m * nf.ldx_next + n] = __float2bfloat16(r * g);
+      float q = live ? r * r : 0.f;          // the 16 lanes of a row: sum of squares over this tile's columns
+      q += __shfl_xor(q, 1, 64);
+      q += __shfl_xor(q, 2, 64);
+      q += __shfl_xor(q, 4, 64);
+      q += __shfl_xor(q, 8, 64);
+      if (c == 0 && m < M) nf.ss_out[(size_t)m * ((gridDim.x + 3) & ~3) + tile] = q;
     }
-    const float rstd = NF ? s_rstd[m < MT * 16 ? m : 0] : 1.f;
-    const float mine = v[j] * rstd;
-    float other = 0.f;
-    if (EPI == EPI_ROPE || EPI == EPI_SWIGLU) other = __shfl_xor(mine, 8, 64);   // the pair's other member
-    if (!live) continue;
-    if (EPI == EPI_ROPE) {
-      const int D = rope.D;
-      const int head = (int)(n / D), jd = (int)(n - (long)head * D);   // column inside the head
-      const int slot = e_slot[j];
-      if (head < rope.Hq + rope.Hkv) {
-        // first member (c < 8): x1 cos - x2 sin; second: x2 cos + x1 sin, x1 being the first member's value
-        const float o = c < 8 ? mine * e_cos[j] - other * e_sin[j] : mine * e_cos[j] + other * e_sin[j];
-        if (head < rope.Hq)
-          ((bf16*)outv)[(size_t)m * ldo + n] = __float2bfloat16(o);
-        else
-          rope.k_cache[(((size_t)(slot / rope.page) * rope.Hkv + (head - rope.Hq)) * rope.page + slot % rope.page) * D + jd] =
-              __float2bfloat16(o);
-      } else {
-        rope.v_cache[(((size_t)(slot / rope.page) * rope.Hkv + (head - rope.Hq - rope.Hkv)) * D + jd) * rope.page +
-                     slot % rope.page] = __float2bfloat16(mine);
-      }
-    } else if (EPI == EPI_STORE_BF16) {
-      ((bf16*)outv)[(size_t)m * ldo + n] = __float2bfloat16(mine);
-    } else if (EPI == EPI_STORE_F32) {
-      ((float*)outv)[(size_t)m * ldo + n] = mine;
-    } else if (c < 8) {                        // SWIGLU: mine = gate, other = up
-      ((bf16*)outv)[(size_t)m * ldo + n] = __float2bfloat16(mine / (1.0f + expf(-mine)) * other);
+    return;
+  }
+  const float rstd = NF ? s_rstd[m] : 1.f;
+  const float mine_v = v * rstd;
+  float other = 0.f;
+  if (EPI == EPI_ROPE || EPI == EPI_SWIGLU) other = __shfl_xor(mine_v, 8, 64);   // the pair's other member
+  if (!live) return;
+  if (EPI == EPI_ROPE) {
+    const int D = rope.D;
+    const int head = (int)(n / D), jd = (int)(n - (long)head * D);   // column inside the head
+    const int slot = e_slot;
+    if (head < rope.Hq + rope.Hkv) {
+      // first member (c < 8): x1 cos - x2 sin; second: x2 cos + x1 sin, x1 being the first member's value
+      const float o = c < 8 ? mine_v * e_cos - other * e_sin : mine_v * e_cos + other * e_sin;
+      if (head < rope.Hq)
+        ((bf16*)outv)[(size_t)m * ldo + n] = __float2bfloat16(o);
+      else
+        rope.k_cache[(((size_t)(slot / rope.page) * rope.Hkv + (head - rope.Hq)) * rope.page + slot % rope.page) * D + jd] =
+            __float2bfloat16(o);
+    } else {
+      rope.v_cache[(((size_t)(slot / rope.page) * rope.Hkv + (head - rope.Hq - rope.Hkv)) * D + jd) * rope.page +
+                   slot % rope.page] = __float2bfloat16(mine_v);
     }
+  } else if (EPI == EPI_STORE_BF16) {
+    ((bf16*)outv)[(size_t)m * ldo + n] = __float2bfloat16(mine_v);
+  } else if (EPI == EPI_STORE_F32) {
+    ((float*)outv)[(size_t)m * ldo + n] = mine_v;
+  } else if (c < 8) {                        // SWIGLU: mine = gate, other = up
+    ((bf16*)outv)[(size_t)m * ldo + n] = __float2bfloat16(mine_v / (1.0f + expf(-mine_v)) * other);
   }
 }
 
 MIE_EXPORT const char* gemm_bf16_last_error() { return g_mie_error; }
-MIE_EXPORT int mie_skinny_max_rows() { return 64; }
+MIE_EXPORT int mie_skinny_max_rows() { return 16; }
 
-template <int MT, int WAVES, bool NF>
+// A kernel that wants more LDS than a launch gets by default is told so once per device.
+static int allow_lds(const void* kernel, int bytes) {
+  static std::mutex lock;
+  static std::set<std::pair<int, const void*>> done;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) MIE_FAIL("skinny_gemm: no current device");
+  std::lock_guard<std::mutex> g(lock);
+  if (done.count({dev, kernel})) return 0;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) MIE_FAIL("skinny_gemm: %d bytes of LDS refused: %s", bytes, hipGetErrorString(e));
+  done.insert({dev, kernel});
+  return 0;
+}
+
+template <bool NF, int SLOTS>
 static int launch_epi(int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx, const bf16* W, long ldw, void* out,
                       long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope, const NormArgs& nf) {
-#define SG_LAUNCH(E)                                                                                               \
-  hipLaunchKernelGGL((skinny_gemm_kernel<MT, E, WAVES, NF>), grid, dim3(WAVES * 64), 0, s, X, ldx, W, ldw, out, ldo, M, \
-                     N, K, up_offset, rope, nf)
+  constexpr int lds = SG_WAVES * SLOTS * RING_U * 2 * 1024;
+#define SG_LAUNCH(E)                                                                                                    \
+  {                                                                                                                     \
+    auto kernel = skinny_gemm_kernel<E, NF, SLOTS>;                                                                     \
+    if (allow_lds((const void*)kernel, lds)) return -1;                                                                 \
+    hipLaunchKernelGGL(kernel, grid, dim3(SG_THREADS), lds, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, nf); \
+  }
   switch (epi) {
     case EPI_STORE_BF16: SG_LAUNCH(EPI_STORE_BF16); break;
     case EPI_STORE_F32: SG_LAUNCH(EPI_STORE_F32); break;
@@ -350,39 +342,38 @@ static int launch_epi(int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx
   return 0;
 }
 
-template <int MT>
-static int launch_waves(int waves, bool fused_norm, int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx,
-                        const bf16* W, long ldw, void* out, long ldo, int M, int N, int K, int up_offset,
-                        const RopeArgs& rope, const NormArgs& nf) {
-#define SG_WAVES_CASE(WV)                                                                                              \
-  if (waves == WV)                                                                                                     \
-    return fused_norm ? launch_epi<MT, WV, true>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, nf) \
-                      : launch_epi<MT, WV, false>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, nf)
-  SG_WAVES_CASE(8);
-  SG_WAVES_CASE(4);
-#undef SG_WAVES_CASE
-  MIE_FAIL("skinny_gemm: %d waves", waves);
+// Slots a wave's ring has.  Four (64 KB a workgroup, two workgroups a compute unit) stream best; three (48 KB,
+// three workgroups a compute unit) when that lets all tiles run at once instead of in two rounds.  Chosen from
+// the weight's shape alone, never from the batch (the sums do not depend on it anyway).
+static int compute_units() {
+  static int units[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!units[dev]) {
+    int n = 0;
+    units[dev] = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256;
+  }
+  return units[dev];
 }
-
-// Waves a tile: the fewer tiles a product has, the more waves share one, so that enough loads are in
-// flight to fill the memory system (16 waves were measured slower than 8 at every shape).  Chosen from
-// the weight's shape alone, never from the batch.
-static int waves_for(int tiles) { return tiles < 256 ? 8 : 4; }
+static int slots_for(int tiles) {
+  const int cu = compute_units();
+  return tiles > 2 * cu && tiles <= 3 * cu ? 3 : 4;
+}
 
 static int launch_rows(int tiles, int epi, hipStream_t s, const bf16* X, long ldx, const bf16* W, long ldw, void* out,
                        long ldo, int M, int N, int K, int up_offset, const RopeArgs& rope, const NormArgs* nf) {
   dim3 grid(tiles);
-  const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  const int waves = waves_for(tiles);
   NormArgs none = {};
   const NormArgs& n = nf ? *nf : none;
-  if (MT == 1) return launch_waves<1>(waves, nf != nullptr, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n);
-  if (MT == 2) return launch_waves<2>(waves, nf != nullptr, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n);
-  return launch_waves<4>(waves, nf != nullptr, epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n);
+  if (slots_for(tiles) == 3)
+    return nf ? launch_epi<true, 3>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n)
+              : launch_epi<false, 3>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n);
+  return nf ? launch_epi<true, 4>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n)
+            : launch_epi<false, 4>(epi, grid, s, X, ldx, W, ldw, out, ldo, M, N, K, up_offset, rope, n);
 }
 
 static int check_operands(const char* what, const void* X, long ldx, const void* W, long ldw, int M, int K) {
-  if (M > 64) MIE_FAIL("%s: %d rows (at most 64)", what, M);
+  if (M > 16) MIE_FAIL("%s: %d rows (at most 16)", what, M);
   if (K <= 0 || (K & 7)) MIE_FAIL("%s: K = %d must be a positive multiple of 8", what, K);
   if (ldx < K || ldw < K || (ldw & 7) || (ldx & 7)) MIE_FAIL("%s: leading dims %ld, %ld for K %d", what, ldx, ldw, K);
   if (((uintptr_t)X | (uintptr_t)W) & 15) MIE_FAIL("%s: operands must be 16-byte aligned", what);

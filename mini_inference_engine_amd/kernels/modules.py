@@ -60,3 +60,7 @@ register_kernel_module("lt_gemm", {
     "mie_lt_is_tuned": [L, L, L, I, I, I, I],
     "mie_lt_tune": [P, L, P, L, P, L, I, I, I, I, P, L, I, I, P, L, P, P, P],
 }, flags=["-L/opt/rocm/lib", "-lhipblaslt", "-Wl,-rpath,/opt/rocm/lib"])
+# stream_read: a measurement for bench.py (the rate at which memory that is only read streams in); no model uses it.
+register_kernel_module("stream_read", {
+    "mie_stream_read": [P, L, P, I, I, P],
+})

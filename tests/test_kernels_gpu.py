@@ -24,9 +24,7 @@ DEV = "cuda"
 @pytest.fixture(scope="module")
 def ops():
     from mini_inference_engine_amd.kernels.hip_backend import HipBackend
-    b16 = HipBackend(torch.bfloat16, DEV)
-    b16.SKINNY_MAX_ROWS = 64          # the kernel's own limit: test all of it, whatever the engine's threshold is
-    return {torch.float32: HipBackend(torch.float32, DEV), torch.bfloat16: b16}
+    return {torch.float32: HipBackend(torch.float32, DEV), torch.bfloat16: HipBackend(torch.bfloat16, DEV)}
 
 
 def tol(dtype):
@@ -146,8 +144,10 @@ def normed(ops, stream, w_norm, eps, rows=None, pending=None):
     return Normed(ops, pending, stream, w_norm, eps, rows)
 
 
-SKINNY_SHAPES = [(1, 64, 176), (7, 200, 331), (16, 2048, 2560), (17, 120, 96), (33, 5632, 2048), (64, 2048, 640),
-                 (8, 176, 64), (3, 96, 384)]
+# (rows, K, N); 9,600 and 12,304 weight rows are 600 and 769 tiles: more than two, and more than three, a compute unit
+# (the kernel's ring is one slot shorter in between); K = 8 and 40: waves without a k-step of their own
+SKINNY_SHAPES = [(1, 64, 176), (7, 200, 331), (16, 2048, 2560), (13, 120, 96), (11, 5632, 2048), (16, 2048, 640),
+                 (8, 176, 64), (3, 96, 384), (5, 264, 9600), (9, 72, 12304), (16, 4104, 48), (2, 8, 32), (6, 40, 16)]
 
 
 @pytest.mark.parametrize("shape", SKINNY_SHAPES)
@@ -339,6 +339,22 @@ def test_projection_kernels_refuse_what_they_cannot_run(engine_ops):
     assert b"splits" in lib._mie_error()
 
 
+def test_few_row_product_refuses_what_it_cannot_run(engine_ops):
+    o = engine_ops
+    lib = o.lib("gemm_bf16")
+    assert lib.mie_skinny_max_rows() == o.SKINNY_MAX_ROWS == 16
+    x = torch.zeros(17, 64, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(32, 64, device=DEV, dtype=torch.bfloat16)
+    y = torch.zeros(17, 32, device=DEV, dtype=torch.bfloat16)
+    call = lambda M, K, ldx: lib.mie_skinny_gemm(x.data_ptr(), ldx, w.data_ptr(), 64, y.data_ptr(), 32, 0, M, 32, K, None, 0, None, 0,
+                                                 None, None, 0, 0.0, None, None)
+    assert call(17, 64, 64) != 0 and b"at most 16" in lib._mie_error()
+    assert call(16, 60, 64) != 0 and b"multiple of 8" in lib._mie_error()
+    assert call(16, 64, 56) != 0 and b"leading dims" in lib._mie_error()
+    assert call(16, 64, 64) == 0
+    assert not o._skinny_ok(x, w, None) and o._skinny_ok(x[:16], w, None)
+
+
 def test_lazy_norm_input_adds_once(ops):
     """A Normed handed to linear: what is pending is added to the stream exactly once, however often it is used."""
     o = ops[torch.bfloat16]
@@ -416,12 +432,13 @@ def test_norm_folded_into_projection_rotary_store(ops):
     torch.testing.assert_close(vc.float(), vc_ref, atol=2e-2, rtol=1e-2)
 
 
-@pytest.mark.parametrize("M, K, inter", [(1, 64, 176), (8, 2048, 5632), (20, 96, 256), (50, 120, 200), (64, 64, 48)])
+@pytest.mark.parametrize("M, K, inter", [(1, 64, 176), (8, 2048, 5632), (12, 96, 256), (16, 120, 200), (9, 64, 48), (4, 136, 4800)])
 def test_skinny_swiglu(ops, M, K, inter):
     o = ops[torch.bfloat16]
     torch.manual_seed(inter)
     w = (torch.randn(2 * inter, K, device=DEV) / math.sqrt(K) * 2).to(torch.bfloat16)
     x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    assert o._skinny_ok(x, w, None), "this shape must take the fused kernel"
     y = o.linear_silu_mul(x, w, inter)
     gu = x.double() @ w.double().T
     # float32 sums of exact products, one rounding (2^-8 relative) at the end
