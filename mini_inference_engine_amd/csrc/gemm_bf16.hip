@@ -66,6 +66,14 @@ template <> struct RingRead<2> {
   }
 };
 
+// The wait of round `it` < SLOTS - 1 (the counter's limit must be a constant of the instruction).
+template <int SLOTS, int IT> struct RingStart {
+  static __device__ __forceinline__ void wait(int it) {
+    if (it == IT) SG_VMCNT((SLOTS - 2 - IT) * RING_U + (IT + 1) * RING_U * 2);
+    else if constexpr (IT + 1 < SLOTS - 1) RingStart<SLOTS, IT + 1>::wait(it);
+  }
+};
+
 enum { EPI_STORE_BF16 = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3, EPI_ROPE = 4 };
 
 // What the rotary epilogue needs beside the product: W is the fused q/k/v projection; the workgroup owns
@@ -142,16 +150,13 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
 
   // What this lane brings in: row lrow (of the weight tile; of x), k-block lkb of every k-step.  And the one
   // result this thread owns after the waves are summed: x row m, column c of the tile.  The gather of x's
-  // rows, if there is one, is the first thing asked for: addresses depend on it.
+  // rows, if there is one, and the positions are the first things asked for: addresses depend on them.
   const int lrow = lane >> 2, lkb = (lane & 3) ^ ((lrow >> 2) & 3);
   const int m = threadIdx.x >> 4, c = threadIdx.x & 15;
   const bool gather = NF && EPI != EPI_ADD && nf.rows;
   const int lsrc = lrow < M ? (gather ? nf.rows[lrow] : lrow) : 0;
   const int msrc = m < M ? (gather ? nf.rows[m] : m) : 0;
 
-  // What the epilogue reads beside the product is asked for next, so that it has arrived long before it is
-  // used and is older than every load of the ring (the counter of loads on their way runs in issue order).
-  // Every load is unconditional, from an address clamped into the operand.
   bool ok;
   const long n = tile_column<EPI>(tile, c, N, up_offset, rope.D, ok);
   const bool live = m < M && ok;
@@ -160,13 +165,49 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
   float e_old = 0.f, e_cos = 0.f, e_sin = 0.f;
   uint32_t e_g = 0u;                       // raw bits of the next norm's weight (converted where it is used)
   int e_slot = 0, e_pos = 0;
+  if (EPI == EPI_ROPE) {                   // the positions: further addresses depend on them too
+    e_pos = rope.positions[mc];
+    e_slot = rope.slots[mc];
+  }
+
+  // The ring.  Slots beyond the wave's range load zeros only, so that it is always filled and drained the
+  // same way.
+  bool lok;
+  const long lwr = tile_column<EPI>(tile, lrow, N, up_offset, rope.D, lok);
+  const bf16* wsrc = W + (size_t)(lok ? lwr : 0) * ldw + lkb * 8;   // a row that does not exist is never stored
+  const bf16* xsrc = X + (size_t)lsrc * ldx + lkb * 8;              // rows beyond M read row 0 along with the lanes that own it
+  const bf16* zero_lane = reinterpret_cast<const bf16*>(mie_zero_words) + lkb * 8;   // per lane, so that choosing it is a select
+  char* mine = ring_lds + wave * WAVE_BYTES;
+  // what: 1 the weight fragments of slot s, 2 the x fragments, 3 both (weight, x, weight, x)
+  auto issue = [&](int s, int what) {
+    char* base = mine + (s % SLOTS) * SLOT_BYTES;
+    const int ks = ks0 + s * RING_U;
+#pragma unroll
+    for (int u = 0; u < RING_U; ++u) {
+      const bool kok = ks + u < ks1 && (ks + u) * 32 + lkb * 8 < K;
+      const bf16* a = kok ? wsrc + (size_t)(ks + u) * 32 : zero_lane;
+      const bf16* b = kok ? xsrc + (size_t)(ks + u) * 32 : zero_lane;
+      if (what & 1)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)a,
+                                         (__attribute__((address_space(3))) void*)(base + (2 * u) * 1024), 16, 0, 0);
+      if (what & 2)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)b,
+                                         (__attribute__((address_space(3))) void*)(base + (2 * u + 1) * 1024), 16, 0, 0);
+    }
+  };
+  const int rounds = ks1 > ks0 ? (ks1 - ks0 + RING_U - 1) / RING_U : 0;
+  // this lane's piece of a fragment: row col, block kb
+  const uint32_t at0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)mine + (col * 4 + (kb ^ ((col >> 2) & 3))) * 16;
+  // The ring starts with the weights of its first slots; their x follows below, after what the epilogue reads
+  // has been asked for: all that waits for the row numbers of a gather, the weights do not.
+#pragma unroll
+  for (int s = 0; s < SLOTS - 1; ++s) issue(s, 1);
+  // What the epilogue reads beside the product is asked for next, so that it has arrived long before it is
+  // used and is older than the ring's x loads (the counter of loads on their way runs in issue order).
+  // Every load is unconditional, from an address clamped into the operand.
   if (EPI == EPI_ADD) {
     e_old = ((const float*)outv)[(size_t)mc * ldo + nc];
     if (NF) e_g = nf.g_f32 ? ((const uint32_t*)nf.g)[nc] : (uint32_t)((const uint16_t*)nf.g)[nc];
-  }
-  if (EPI == EPI_ROPE) {
-    e_pos = rope.positions[mc];
-    e_slot = rope.slots[mc];
   }
   // Fused norm, consuming side: the partial sums of squares likewise.  16 lanes a row, lane c takes the
   // tiles 4 (c + 16 i) .. + 3: the first SSP fours now, the rest (widths above 4096) after the loop.
@@ -181,32 +222,9 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
     }
   }
 
-  // The ring.  Slots beyond the wave's range load zeros only, so that it is always filled and drained the
-  // same way.
-  bool lok;
-  const long lwr = tile_column<EPI>(tile, lrow, N, up_offset, rope.D, lok);
-  const bf16* wsrc = W + (size_t)(lok ? lwr : 0) * ldw + lkb * 8;   // a row that does not exist is never stored
-  const bf16* xsrc = X + (size_t)lsrc * ldx + lkb * 8;              // rows beyond M read row 0 along with the lanes that own it
-  const bf16* zero_lane = reinterpret_cast<const bf16*>(mie_zero_words) + lkb * 8;   // per lane, so that choosing it is a select
-  char* mine = ring_lds + wave * WAVE_BYTES;
-  auto issue = [&](int s) {
-    char* base = mine + (s % SLOTS) * SLOT_BYTES;
-    const int ks = ks0 + s * RING_U;
+  // the x fragments of the ring's first slots
 #pragma unroll
-    for (int u = 0; u < RING_U; ++u) {
-      const bool kok = ks + u < ks1 && (ks + u) * 32 + lkb * 8 < K;
-      const bf16* a = kok ? wsrc + (size_t)(ks + u) * 32 : zero_lane;
-      const bf16* b = kok ? xsrc + (size_t)(ks + u) * 32 : zero_lane;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)a,
-                                       (__attribute__((address_space(3))) void*)(base + (2 * u) * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)b,
-                                       (__attribute__((address_space(3))) void*)(base + (2 * u + 1) * 1024), 16, 0, 0);
-    }
-  };
-  const int rounds = ks1 > ks0 ? (ks1 - ks0 + RING_U - 1) / RING_U : 0;
-  // this lane's piece of a fragment: row col, block kb
-  const uint32_t at0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)mine + (col * 4 + (kb ^ ((col >> 2) & 3))) * 16;
-  for (int s = 0; s < SLOTS - 1; ++s) issue(s);
+  for (int s = 0; s < SLOTS - 1; ++s) issue(s, 2);
   if (EPI == EPI_ROPE) {
     // the angles, once the positions are here (asked for before the ring: waiting for them does not wait for it)
     const int half = rope.D >> 1;
@@ -217,8 +235,12 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
   }
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int it = 0; it < rounds; ++it) {
-    issue(it + SLOTS - 1);                         // into the slot that was read a round ago
-    SG_VMCNT((SLOTS - 1) * L);                     // slot `it` has landed (anything asked for in between only makes this wait for more)
+    issue(it + SLOTS - 1, 3);                      // into the slot that was read a round ago
+    // Slot `it` has landed: all but the loads issued after its last one.  From round SLOTS - 1 on those are the
+    // SLOTS - 1 slots after it; before, the x fragments of the first slots that follow its own and the slots
+    // issued in the loop so far.  (Anything else asked for in between only makes this wait for more.)
+    if (it >= SLOTS - 1) SG_VMCNT((SLOTS - 1) * L);
+    else RingStart<SLOTS, 0>::wait(it);
     sg_u32x4 f[2 * RING_U];
     RingRead<RING_U>::run(at0 + (it % SLOTS) * SLOT_BYTES, f);
 #pragma unroll

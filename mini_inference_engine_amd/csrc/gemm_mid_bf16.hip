@@ -6,10 +6,14 @@
 //   part[s, m, n] = sum over the k of split s of x[m, k] W[n, k]
 //
 // a workgroup of 4 waves owns 64 weight rows and one contiguous range of K (the split); k-steps of W
-// and of x (all rows) are brought into a ring of LDS stages by loads that write the LDS directly, every
-// fragment already in the order the matrix instruction wants it (1 KB a fragment, lane l at 16 l), so
-// x is read once per 64 weight rows and the fragment reads are conflict-free; wave w multiplies its 16
-// weight rows with v_mfma_f32_16x16x32_bf16.  The split's sums go out as float32 partial results.
+// and of x (all rows) are brought into a ring of LDS stages by loads that write the LDS directly, 1 KB a
+// fragment (16 rows x 32 k), so x is read once per 64 weight rows; wave w multiplies its 16 weight rows
+// with v_mfma_f32_16x16x32_bf16.  The split's sums go out as float32 partial results.
+// A fragment is brought in by lane 4 r + b reading k-block b ^ (r / 4) % 4 of row r (16 bytes): a quarter
+// wave then reads 64 contiguous bytes of 4 rows (in the matrix instruction's own order, lane 16 b + r, it
+// touches 16 cache lines for 16 bytes each, and the address unit's line look-ups bound the kernel), and the
+// permutation of the blocks spreads the fragment reads (lane 16 b + r reads slot 4 r + (b ^ (r / 4) % 4))
+// over all banks.
 // The number of splits is chosen by the caller from the weight's shape alone, so a row's result does
 // not depend on the batch it is in.
 //
@@ -112,35 +116,38 @@ mid_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict__ W
   static_assert((MID_STAGES - 2) * L <= 63, "more loads in flight than the counter holds");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kb = lane >> 4;
+  const int lrow = lane >> 2, lkb = (lane & 3) ^ ((lrow >> 2) & 3);     // the row and k-block this lane brings in
+  const int rslot = col * 4 + (kb ^ ((col >> 2) & 3));                  // where this lane's piece of a fragment sits
   const int ksteps = (K + 31) >> 5;
   const int ksA = blockIdx.y * kper, ksB = ksA + kper < ksteps ? ksA + kper : ksteps;
   const int nst = (ksB - ksA + MID_KC - 1) / MID_KC;
   const int n = (blockIdx.x * MID_WAVES + wave) * 16 + col;
-  const bf16* wrow = W + (size_t)(n < N ? n : N - 1) * ldw + kb * 8;
+  const int nl = (blockIdx.x * MID_WAVES + wave) * 16 + lrow;
+  const bf16* wrow = W + (size_t)(nl < N ? nl : N - 1) * ldw + lkb * 8;
   const bf16* xptr[XL];
   int xkc[XL], xlds[XL];
 #pragma unroll
   for (int j = 0; j < XL; ++j) {
     const int f = wave * XL + j, kc = f / MT, mt = f % MT;
-    const int m = mt * 16 + col;
-    xptr[j] = X + (size_t)(m < M ? m : 0) * ldx + kc * 32 + kb * 8;
+    const int m = mt * 16 + lrow;
+    xptr[j] = X + (size_t)(m < M ? m : 0) * ldx + kc * 32 + lkb * 8;
     xkc[j] = kc;
     xlds[j] = (kc * SF + MID_WAVES + mt) * FRAG_BYTES;
   }
-  const bf16* zero_lane = zeros + kb * 8;      // a per-lane address, so that choosing it is a select and no branch
+  const bf16* zero_lane = zeros + lkb * 8;     // a per-lane address, so that choosing it is a select and no branch
   auto issue = [&](int s) {
     char* base = lds + (s % MID_STAGES) * STAGE_BYTES;
     const int ks = ksA + s * MID_KC;
 #pragma unroll
     for (int kc = 0; kc < MID_KC; ++kc) {
-      const bool ok = ks + kc < ksB && (ks + kc) * 32 + kb * 8 < K;
+      const bool ok = ks + kc < ksB && (ks + kc) * 32 + lkb * 8 < K;
       const bf16* src = ok ? wrow + (size_t)(ks + kc) * 32 : zero_lane;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(base + (kc * SF + wave) * FRAG_BYTES), 16, 0, 0);
     }
 #pragma unroll
     for (int j = 0; j < XL; ++j) {
-      const bool ok = ks + xkc[j] < ksB && (ks + xkc[j]) * 32 + kb * 8 < K;
+      const bool ok = ks + xkc[j] < ksB && (ks + xkc[j]) * 32 + lkb * 8 < K;
       const bf16* src = ok ? xptr[j] + (size_t)ks * 32 : zero_lane;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(base + xlds[j]), 16, 0, 0);
@@ -156,7 +163,7 @@ mid_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict__ W
     MID_VMCNT((MID_STAGES - 2) * L);           // this wave's loads of stage `it` have landed
     __builtin_amdgcn_s_barrier();              // and everybody else's; everybody is done reading stage it - 1
     issue(it + MID_STAGES - 1);                // into the buffer stage it - 1 used
-    const uint32_t base = lds0 + (it % MID_STAGES) * STAGE_BYTES + lane * 16;
+    const uint32_t base = lds0 + (it % MID_STAGES) * STAGE_BYTES + rslot * 16;
     StageReader<MT, 0>::run(base, base + wave * FRAG_BYTES, acc);
   }
   MID_VMCNT(0);                                // nothing of this wave may still be writing the LDS when it ends
