@@ -111,7 +111,7 @@ def measured_peaks() -> dict:
     words = torch.empty(8192 * 256, dtype=torch.int32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
     t_read = min(best(lambda: library.check(reader, reader.mie_stream_read(src.data_ptr(), src.numel(), words.data_ptr(), groups, nt, stream)))
-                 for nt in (0, 1) for groups in (1024, 2048, 4096, 8192))
+                 for nt in (0, 1) for groups in (512, 768, 1024, 2048, 4096))
     del src, dst, words
     a = torch.randn(8192, 8192, device="cuda").to(torch.bfloat16)
     b = torch.randn(8192, 8192, device="cuda").to(torch.bfloat16)
