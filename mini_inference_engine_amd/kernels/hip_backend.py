@@ -198,9 +198,8 @@ class HipBackend(KernelBackend):
         return y
 
     # ---- few-row products of the bfloat16 path: one fused kernel each
-    SKINNY_MAX_ROWS = 16      # above this the split product or the library is faster than the fused kernel (decode steps of the
-                              # benchmark's sizes: 16 rows 1.24 against 1.28 ms; 24 rows 1.40 against 1.29; 32 rows 1.55 against 1.32;
-                              # the same crossing at the layer sizes of Llama-2-7B and Llama-3-8B)
+    SKINNY_MAX_ROWS = 16      # the kernel's own limit (one tile of rows); a decode step of 16 rows of 512 keys at the
+                              # benchmark's sizes takes 1.15 ms, one of 17 rows with the split product 1.27
     EPI_BF16, EPI_F32, EPI_ADD, EPI_SWIGLU = 0, 1, 2, 3
 
     def _skinny_ok(self, x, w, bias, rows=None) -> bool:
