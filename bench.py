@@ -320,7 +320,8 @@ def measure_kernels(cfg, args) -> int:
     w = weights(h, inter)
     t = timed(lambda i: ops.linear(act, w[i % copies], add_to=Sink(stream, g_norm, cfg.rms_norm_eps)), copies)
     report(f"down product + add + next norm, {M} rows", t, 2 * h * inter + M * (2 * inter + 8 * h + 2 * h))
-    w = weights(V, h)[:max(2, copies // 4)]
+    # the head's weights: sets enough for twice the 256 MB memory-side cache
+    w = [(torch.randn(V, h, device=dev) * 0.02).to(torch.bfloat16) for _ in range(max(2, -(-(512 << 20) // (V * h * 2))))]
     t = timed(lambda i: ops.linear(x, w[i % len(w)], out_dtype=torch.float32), len(w))
     report(f"head product, float32 logits, {M} rows", t, 2 * V * h + M * (2 * h + 4 * V))
     del w
