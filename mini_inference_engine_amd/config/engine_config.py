@@ -25,6 +25,7 @@ class EngineConfig:
     num_state_slots: int | None = None      # default: max_num_seqs + 1 (slot 0 is scratch)
     use_hip_graphs: bool = True
     graph_batch_sizes: tuple = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 160, 192, 224, 256)
+    portion_graph_sizes: tuple | None = None   # token counts of the captured single-prompt steps; None: eighths of the token budget
     seed: int = 0                           # base of every request's sampling stream
     activation_reserve_bytes: int = 768 * 2**20
     poison_freed_pages: bool = False        # debugging: fill returned pages with NaN
@@ -57,4 +58,6 @@ class EngineConfig:
         values.update(overrides)
         if "graph_batch_sizes" in values:
             values["graph_batch_sizes"] = tuple(values["graph_batch_sizes"])
+        if values.get("portion_graph_sizes") is not None:
+            values["portion_graph_sizes"] = tuple(values["portion_graph_sizes"])
         return cls(**values)

@@ -122,9 +122,12 @@ def order_rows(rows: Sequence[StepRow]) -> list[int]:
 
 
 def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad_rows_to: int = 0,
-               static_context: int = 0, want_all: bool = False, sampling=None) -> StepContext:
+               static_context: int = 0, want_all: bool = False, sampling=None, pad_portion_to: int = 0) -> StepContext:
     """Flatten ``rows`` into ``arena``.  ``pad_rows_to`` adds scratch rows (one token at
-    position 0, page 0, slot 0) up to a captured batch size.  ``want_all`` asks for the logits
+    position 0, page 0, slot 0) up to a captured batch size.  ``pad_portion_to`` (one row only) lengthens the
+    row to a captured number of tokens: token 0 at the positions that follow, written to the scratch page, which
+    is also what the row's block table names beyond its own pages; no token of the row itself looks at them (they
+    come later), and what they compute is nobody's.  ``want_all`` asks for the logits
     of every token in flat order (what a captured step produces) instead of the rows' wants.
     ``sampling``: (temperatures, seeds, counters), one entry for each wanted row of logits in their order
     (with ``want_all``: one for each of ``rows``; scratch rows are greedy), for a step whose tokens are
@@ -133,6 +136,10 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
     order = order_rows(rows)
     n_rows = len(rows)
     lens = np.fromiter((len(rows[i].tokens) for i in order), dtype=np.int64, count=n_rows)
+    if pad_portion_to:
+        if n_rows != 1 or pad_rows_to or pad_portion_to < lens[0]:
+            raise ValueError(f"padding to {pad_portion_to} tokens is for one row of at most as many, without padding rows")
+        lens[0] = pad_portion_to
     total_rows = max(n_rows, pad_rows_to)
     if total_rows == 0 or (lens <= 0).any():
         raise ValueError("a step needs at least one row and every row at least one token")
@@ -175,7 +182,9 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
                 ids[a] = 0
                 taken[a] = rows[i].taken_from
             else:
-                ids[a:b] = rows[i].tokens
+                real = len(rows[i].tokens)
+                ids[a:a + real] = rows[i].tokens
+                ids[a + real:b] = 0
             slots_state[r] = rows[i].cache.state_slot
             new_row_of[i] = r
     arena.host_view("positions")[:T] = positions
@@ -215,11 +224,13 @@ def build_step(rows: Sequence[StepRow], arena: StepArena, page_size: int, *, pad
             if i is None:
                 continue
             t = rows[i].cache.tables[g]
-            need = -(-int(ctx[r]) // page_size)
+            need = -(-int(row_pos[r] + (len(rows[i].tokens) if pad_portion_to else row_len[r])) // page_size)
             if len(t) < need:
                 raise ValueError(f"row {i}: {len(t)} pages reserved in group {g}, {need} needed")
             bt[r, :need] = t[:need]
         page_of = bt[token_row, positions // page_size].astype(np.int64)
+        if pad_portion_to:                              # padding tokens: the scratch page, also where the row's last page has room
+            page_of[len(rows[0].tokens):] = 0
         arena.host_view(f"slot_mapping{g}")[:T] = page_of * page_size + positions % page_size
 
     arena.upload(total_rows)

@@ -1,5 +1,5 @@
-"""Captured steps: one hipGraph per batch-size bucket of single-token rows, and one for a prompt portion of
-exactly the step's token budget.
+"""Captured steps: one hipGraph per batch-size bucket of single-token rows, and one per size for a step that
+holds a single prompt portion.
 
 A step of single-token rows is launch-bound when run kernel by kernel.  As in the
 reference (inference_engine/engine.py:76-120), the whole forward of such a step is
@@ -12,8 +12,12 @@ upload.  No memset node is recorded: buffers are cleared by kernels.
 A long prompt comes in portions of exactly the token budget of a step; such a step (one row, that many tokens,
 starting anywhere in its request, at most one position whose logits are wanted) has the same launches every time
 and is captured too (PortionGraph): launched kernel by kernel it costs the host about 3 ms, of which half a
-millisecond is not hidden behind the device when the engine was idle.  The reference captures single-token steps
-only.
+millisecond is not hidden behind the device when the engine was idle.  A shorter prompt, or the rest of a long
+one, runs in the smallest captured size that holds it (the entry point captures eighths of the budget), lengthened
+with padding tokens: token 0 at the positions that follow, written to the scratch page, which no token of the
+prompt itself looks at since they come later; a 512-token prompt then takes what its kernels take instead of what
+its launches take.  Not for a model with a mixer whose state every token of a row changes.  The reference captures
+single-token steps only.
 """
 from __future__ import annotations
 
@@ -99,7 +103,9 @@ class _ScratchRequest:
 
 
 class PortionGraph:
-    """The captured step of one row of exactly ``tokens`` tokens with one row of logits."""
+    """The captured step of one row of ``tokens`` tokens with one row of logits.  It runs a prompt portion of
+    exactly that many tokens, or, where the model allows padding tokens (``Decoder.padding_safe``), a shorter
+    one lengthened to it."""
 
     def __init__(self, runner, tokens: int, pool=None):
         from .batch import StepRow
@@ -122,9 +128,12 @@ class PortionGraph:
                 gc.enable()
         torch.cuda.synchronize()
 
-    def takes(self, rows) -> bool:
-        return (len(rows) == 1 and len(rows[0].tokens) == self.tokens and len(rows[0].want) <= 1
-                and rows[0].taken_from < 0)
+    def takes(self, rows, padding_safe: bool = False) -> bool:
+        if len(rows) != 1 or len(rows[0].want) > 1 or rows[0].taken_from >= 0:
+            return False
+        n = len(rows[0].tokens)
+        return n == self.tokens or (padding_safe and 2 <= n < self.tokens
+                                    and rows[0].start + self.tokens <= self.static_context)
 
     def run(self, runner, rows, sampling=None):
         """Logits [1, vocab] of the row's wanted position (None if it wants none), and the step as built."""
@@ -132,8 +141,9 @@ class PortionGraph:
         row = rows[0]
         wanted = bool(len(row.want))
         if not wanted:                                  # the graph computes one row of logits whatever happens: the last token's
-            row = StepRow(row.cache, row.tokens, row.start, [self.tokens - 1])
-        step = runner.build([row], static_context=self.static_context, sampling=sampling if wanted else None)
+            row = StepRow(row.cache, row.tokens, row.start, [len(row.tokens) - 1])
+        step = runner.build([row], static_context=self.static_context, sampling=sampling if wanted else None,
+                            pad_portion_to=self.tokens)
         with runner.ranges("forward"):
             self.graph.replay()
         return (self.logits if wanted else None), step

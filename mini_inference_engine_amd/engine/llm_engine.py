@@ -84,8 +84,12 @@ class LLMEngine:
             self.tokenizer = AutoTokenizer.from_pretrained(model)
         if cfg.use_hip_graphs and self.runner.device.type == "cuda":
             self.runner.capture_decode_graphs(cfg.graph_batch_sizes, verbose=verbose, sample=True)
-            if cfg.enable_chunked_prefill and 2 <= cfg.max_num_batched_tokens <= self.runner.max_model_len:
-                self.runner.capture_portion_graph(cfg.max_num_batched_tokens)
+            sizes = cfg.portion_graph_sizes
+            if sizes is None:           # eighths of the token budget: a prompt runs in a step at most an eighth of it longer
+                most = min(cfg.max_num_batched_tokens, self.runner.max_model_len)
+                sizes = sorted({most * k // 8 for k in range(1, 9) if most * k // 8 >= 64} | ({most} if most >= 2 else set()))
+            if cfg.enable_chunked_prefill and sizes:
+                self.runner.capture_portion_graphs(sizes)
         self.graphs = self.runner.graphs
         self.num_steps = 0
         self.num_graph_steps = 0

@@ -104,7 +104,7 @@ class ModelRunner:
         # from here on the device (StepRow.taken_from) before the host has seen it.
         self.chosen_tokens = torch.zeros(max(1, max_rows), dtype=torch.int32, device=self.device)
         self.graphs = None                  # captured decode steps, once capture_decode_graphs was called
-        self.portion_graph = None           # the captured step of one full-budget prompt portion (capture_portion_graph)
+        self.portion_graphs = []            # captured steps of one prompt portion, by token count (capture_portion_graphs)
         self.last_step_captured = False
         self.ranges = PhaseRanges(False)    # the entry point switches them on (EngineConfig.trace_ranges)
 
@@ -131,18 +131,31 @@ class ModelRunner:
             self.ops.prefer_rows(batch_sizes)     # these row counts recur: the warm-up before each capture may choose kernels
         self.graphs = DecodeGraphs(self, batch_sizes, verbose=verbose, sample=sample)
 
-    def capture_portion_graph(self, tokens: int | None = None) -> None:
-        """Capture the step that holds one prompt portion of exactly ``tokens`` tokens (default: the step's token
-        budget, what a long prompt is cut into); ``forward_step`` replays it for such steps."""
+    def capture_portion_graphs(self, sizes=None) -> None:
+        """Capture the step that holds one prompt portion, once for each token count in ``sizes`` (default: the
+        step's token budget, what a long prompt is cut into); ``forward_step`` replays the smallest that holds
+        such a step: a portion of exactly that many tokens, or, if the model allows padding tokens, a shorter one."""
         from .graphs import PortionGraph
-        tokens = int(tokens or self.arena.max_tokens)
-        if not 2 <= tokens <= min(self.arena.max_tokens, self.max_model_len):
-            raise ValueError(f"a captured portion of {tokens} tokens does not fit a step of {self.arena.max_tokens} "
-                             f"or a request of {self.max_model_len}")
+        most = min(self.arena.max_tokens, self.max_model_len)
+        sizes = sorted({int(t) for t in (sizes or [self.arena.max_tokens])})
+        if not sizes or sizes[0] < 2 or sizes[-1] > most:
+            raise ValueError(f"captured portions of {sizes} tokens: between 2 and {most} (the step's budget, the "
+                             f"longest request)")
         if self.tune_library_products:
-            self.ops.prefer_rows([tokens])
+            self.ops.prefer_rows(sizes[-1:])          # the budget's own size recurs with every long prompt
         pool = next(iter(self.graphs.graphs.values()))[0].pool() if self.graphs is not None and self.graphs.graphs else None
-        self.portion_graph = PortionGraph(self, tokens, pool=pool)
+        self.portion_graphs = []
+        for tokens in reversed(sizes):                # the largest first: the others fit into what it reserved
+            self.portion_graphs.append(PortionGraph(self, tokens, pool=pool))
+            if pool is None:
+                pool = self.portion_graphs[0].graph.pool()
+        self.portion_graphs.reverse()
+
+    def _portion_graph_for(self, rows):
+        for g in self.portion_graphs:
+            if g.takes(rows, self.model.padding_safe):
+                return g
+        return None
 
     @torch.inference_mode()
     def forward_step(self, rows: list[StepRow], sampling=None) -> torch.Tensor | None:
@@ -156,9 +169,10 @@ class ModelRunner:
         self.last_step_captured = False
         captured = (self.graphs is not None and self.graphs.fits(len(rows)) and all(len(r.tokens) == 1 for r in rows)
                     and (sampling is None or all(len(r.want) == 1 for r in rows)))
-        if not captured and self.portion_graph is not None and self.portion_graph.takes(rows):
+        portion = None if captured or not self.portion_graphs else self._portion_graph_for(rows)
+        if portion is not None:
             self.last_step_captured = True
-            logits, step = self.portion_graph.run(self, rows, sampling)
+            logits, step = portion.run(self, rows, sampling)
         elif captured:
             self.last_step_captured = True
             logits, step = self.graphs.run(self, rows, sampling)

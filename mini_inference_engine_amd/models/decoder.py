@@ -45,6 +45,9 @@ class Decoder:
                 ce.group = group_keys.index(key)
             self.cache_entries[e] = ce
         self.bindings: list[CacheBinding] = []
+        # whether a step may carry padding tokens (written to the scratch page): not if a mixer keeps state that
+        # every token of a row changes
+        self.padding_safe = all(ce.requirement.paged for ce in self.cache_entries.values())
 
     # ------------------------------------------------------------ structure
     def parts(self):

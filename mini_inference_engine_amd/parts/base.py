@@ -138,7 +138,9 @@ class CacheRequirement:
     keys and values, several state tensors) is a subclass; nothing else changes.
 
     paged        True: data per token, in pages that the cache manager hands out per request; requirements
-                 with equal ``page_group_key()`` share page ids and block tables.
+                 with equal ``page_group_key()`` share page ids and block tables.  What a token writes goes to its
+                 slot only, so a step may carry padding tokens that write to the scratch page (a model all of
+                 whose requirements are paged can run a prompt portion in a captured step of more tokens).
     window       for paged data: how many keys back a query looks at most (None = all); pages that lie
                  wholly before the window are given back.
     bytes_per_page(page_size, element_size)   what one page id costs in this entry (sizes the pool)

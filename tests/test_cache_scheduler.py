@@ -275,3 +275,36 @@ def test_random_workloads_finish_with_all_pages_back(seed):
         assert steps < 5000
     assert all(s.status is Status.FINISHED and s.num_output_tokens == s.params.max_tokens for s in seqs)
     assert cm.num_free(0) == cm.usable_pages(0) and not cm.live
+
+
+# ------------------------------------------------------------------------------- a step's arrays
+def test_a_portion_lengthened_to_a_captured_size_writes_to_the_scratch_page():
+    """build_step(pad_portion_to=N): the row's own tokens keep their ids, positions and slots; the padding
+    tokens follow at the next positions with id 0, their slots lie in page 0, and the block table names page 0
+    beyond the row's own pages."""
+    import numpy as np
+    import torch
+    from types import SimpleNamespace
+    from mini_inference_engine_amd.engine.batch import StepArena, StepRow, build_step
+    page = 4
+    arena = StepArena(32, 4, 16, 1, torch.device("cpu"))
+    req = SimpleNamespace(tables=[[7, 3, 9]], state_slot=2)             # positions 0 .. 11
+    step = build_step([StepRow(req, [11, 12, 13, 14, 15], 5, [4])], arena, page, pad_portion_to=16, static_context=64)
+    assert step.num_tokens == 16 and step.num_rows == 1 and step.num_decode_rows == 0 and step.max_context == 64
+    assert step.input_ids.tolist() == [11, 12, 13, 14, 15] + [0] * 11
+    assert step.positions.tolist() == list(range(5, 21))
+    assert step.logit_rows.tolist() == [4]
+    slots = arena.dev_view("slot_mapping0", 16).tolist()
+    assert slots[:5] == [3 * page + 1, 3 * page + 2, 3 * page + 3, 9 * page + 0, 9 * page + 1]
+    assert all(0 <= s < page for s in slots[5:]), "padding tokens write to page 0"
+    table = arena.dev_view("block_tables0", 16).tolist()
+    assert table[:3] == [7, 3, 9] and table[3:6] == [0, 0, 0]
+    assert step.host["row_context"].tolist() == [21]
+    # positions 5 .. 9 need three pages; two are not enough, padding or not
+    short = SimpleNamespace(tables=[[7, 3]], state_slot=0)
+    with pytest.raises(ValueError, match="pages reserved"):
+        build_step([StepRow(short, [1, 2, 3, 4, 5], 5, [])], arena, page, pad_portion_to=16)
+    with pytest.raises(ValueError, match="one row"):
+        build_step([StepRow(req, [1, 2], 0, []), StepRow(req, [3, 4], 2, [])], arena, page, pad_portion_to=16)
+    with pytest.raises(ValueError, match="one row"):
+        build_step([StepRow(req, list(range(9)), 0, [])], arena, page, pad_portion_to=8)

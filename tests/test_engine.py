@@ -339,28 +339,35 @@ def test_tokens_chosen_in_the_step_gpu(tiny_models, capture):
 def test_full_budget_portions_through_the_captured_graph(tiny_models, dtype):
     """A prompt longer than the step's token budget comes in portions of exactly the budget; that step is
     captured once and replayed (wherever in the request the portion starts, whether or not its logits are
-    wanted).  The same portions launched kernel by kernel by a second runner must give the same logits, bit for
-    bit in float32; then generation through the entry point, which reaches the graph by itself."""
+    wanted).  A shorter portion runs in the smallest captured step that holds it, lengthened with padding tokens
+    that write to the scratch page; one that would reach beyond the longest request that way, or that wants two
+    rows of logits, is launched kernel by kernel.  The same portions launched kernel by kernel by a second runner
+    must give the same logits, bit for bit in float32; then generation through the entry point, which reaches
+    the graphs by itself."""
     from mini_inference_engine_amd.engine.batch import StepRow
     from mini_inference_engine_amd.engine.runner import ModelRunner
     m = tiny_models["B"]
     folder = m["folder_f32"] if dtype == "float32" else m["folder_bf16"]
     budget = 48
-    toks = prompts_for(m, [230], seed=9)[0]
+    toks = prompts_for(m, [256], seed=9)[0]
     runners = [ModelRunner(folder, dtype=dtype, device="cuda", num_pages=40, max_rows=4, max_step_tokens=budget)
                for _ in range(2)]
-    runners[0].capture_portion_graph()
+    runners[0].capture_portion_graphs([16, budget])
+    assert [g.tokens for g in runners[0].portion_graphs] == [16, budget] and runners[0].model.padding_safe
     caches = [r.cache.open("a") for r in runners]
     exact = plain_llama.forward(m["cfg"], m["weights"] if dtype == "float32" else m["weights_bf16"], toks)
     start = 0
-    for n, want in ((budget, [budget - 1]), (7, [6]), (budget, []), (budget, [3]), (budget, [budget - 1]), (budget, [0, 1])):
+    # (tokens, wanted offsets, the captured size that runs it); the request may reach position 256
+    for n, want, size in ((budget, [budget - 1], 48), (7, [6], 16), (budget, [], 48), (20, [19], 48), (budget, [3], 48),
+                          (16, [15], 16), (2, [], 16), (17, [5], 48), (30, [0, 1], None), (12, [11], 16), (8, [7], None)):
         outs = []
         for r, rc in zip(runners, caches):
             assert r.cache.reserve(rc, start, n)
             out = r.forward_step([StepRow(rc, toks[start:start + n], start, want)])
             outs.append(None if out is None else out.clone())
-        replayed = n == budget and len(want) <= 1
-        assert runners[0].last_step_captured == replayed and not runners[1].last_step_captured
+        assert runners[0].last_step_captured == (size is not None) and not runners[1].last_step_captured, (start, n)
+        if size is None and len(want) <= 1:
+            assert start + 16 > 256, "only what would reach beyond the longest request is launched kernel by kernel"
         if want:
             if dtype == "float32":
                 assert torch.equal(outs[0], outs[1]), f"portion at {start}: the captured step differs from the launched one"
@@ -370,9 +377,11 @@ def test_full_budget_portions_through_the_captured_graph(tiny_models, dtype):
         else:
             assert outs[0] is None and outs[1] is None
         start += n
+    assert start == 256
     # through the entry point: a prompt of 150 tokens under a budget of 48 is three captured portions and a rest
-    eng = engine(m, "cuda", dtype, num_blocks=40, max_num_seqs=4, max_num_batched_tokens=budget, graph_batch_sizes=(1, 2))
-    assert eng.runner.portion_graph is not None
+    eng = engine(m, "cuda", dtype, num_blocks=40, max_num_seqs=4, max_num_batched_tokens=budget, graph_batch_sizes=(1, 2),
+                 portion_graph_sizes=(budget,))
+    assert [g.tokens for g in eng.runner.portion_graphs] == [budget]
     prompts = prompts_for(m, [150], seed=10)
     sp = SamplingParams(max_tokens=5, ignore_eos=True)
     outs = eng.generate(prompts, sp)
