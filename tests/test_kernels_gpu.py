@@ -639,6 +639,38 @@ def test_decode_attention_past_4096_keys(ops, case, splits, spiked):
         torch.testing.assert_close(out[0].float(), v_far, atol=3e-2, rtol=3e-2)
 
 
+@pytest.mark.parametrize("edge", [None, "first key inside", "last key outside"])
+@pytest.mark.parametrize("window", [1024, 4000])
+@pytest.mark.parametrize("geom", [(32, 8, 128), (32, 4, 64)])
+def test_windowed_attention_at_long_contexts(ops, geom, window, edge):
+    """A window of 1,024 or 4,000 keys at contexts of thousands, at the head sizes and groupings of the benchmark
+    configurations (no registered architecture has a window: the part and the kernels do): single-token rows,
+    where the context bound a kernel is given shrinks to the window, and a portion of 300 tokens behind 5,000
+    earlier ones.  With ``edge``, the key just inside (or just outside) the window of the first row's last query
+    is made to dominate it: inside, its value is what comes out; outside, it must leave no trace."""
+    Hq, Hkv, D = geom
+    dtype = torch.bfloat16
+    for ctx, qn in (([6000, 700, 4096, 1025, 1024, 33], [1] * 6), ([5300, 2100], [300, 40])):
+        spike = None
+        if edge is not None:
+            last = ctx[0] - 1                                        # position of the first row's last query
+            key = last - window + 1 if edge == "first key inside" else last - window
+            spike = (0, key)
+        q, kc, vc, group, step = paged_setup(ctx, qn, Hq, Hkv, D, 16, dtype, seed=D + window + len(ctx), spike=spike)
+        scale = 1 / math.sqrt(D) if edge is None else 1.0
+        out, expect = run_attention(ops, dtype, q, kc, vc, group, step, Hq, Hkv, D, scale, window)
+        torch.testing.assert_close(out.double(), expect, **(ATT_TOL if edge is None else SPIKE_TOL)[dtype])
+        if edge is not None:
+            t_last = qn[0] - 1
+            pg = int(group.block_tables[0, spike[1] // 16])
+            v_key = vc[pg, :, :, spike[1] % 16].float().repeat_interleave(Hq // Hkv, dim=0).reshape(-1)
+            gap = (out[t_last].float() - v_key).abs().max()
+            if edge == "first key inside":
+                assert float(gap) < 3e-2, f"the key at the window's edge should dominate (off by {float(gap):.2e})"
+            else:
+                assert float(gap) > 0.5, "a key one past the window was seen"
+
+
 @pytest.mark.parametrize("key", [None, 5, 6143, 6144, 8100])
 @pytest.mark.parametrize("geom", [(32, 8, 128), (32, 4, 64)])
 def test_prefill_attention_with_6144_earlier_tokens(ops, geom, key):
