@@ -12,7 +12,6 @@ time K steps between device synchronisations.  Prints one JSON line:
   value     decoded tokens a second at ``batch`` (default 8) with contexts just below ``context``
   points    the same at batch 1 and 64, and at ``batch`` with contexts of 512; output and total tokens a second
             of the reference's mixed end-to-end workload (256 requests at once, prompts of 128..512 and outputs
-            of 64..512 tokens; TinyLlama sizes only)
             of 64..512 tokens; TinyLlama sizes only); prompts of 512, 4,096 and 8,192 tokens run in portions of at
             most 2,048 (tokens a second over the whole prompt), and the last such portion of the longest alone
             (2,048 new tokens behind 6,144 earlier ones)
@@ -265,6 +264,7 @@ def measure_kernels(cfg, args) -> int:
     copies = max(2, min(12, int(3e8 // (2 * inter * h * 2)) + 1))     # enough weight sets to exceed every cache
 
     def timed(run, n):
+        n = max(n, 16)                  # launches a graph: few of them would carry the graph's own launch in their time
         run(0)
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
