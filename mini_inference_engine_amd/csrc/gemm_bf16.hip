@@ -31,7 +31,6 @@
 #include "common.hpp"
 #include <mutex>
 #include <set>
-#include <stdlib.h>
 #include <utility>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
