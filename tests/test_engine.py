@@ -387,3 +387,18 @@ def test_full_budget_portions_through_the_captured_graph(tiny_models, dtype):
     outs = eng.generate(prompts, sp)
     assert eng.num_graph_steps >= 3 + 4, "three portions and the single-token steps after them must have been replayed"
     check_outputs(m, prompts, outs, [sp], 1e-5 if dtype == "float32" else 2e-2, "weights" if dtype == "float32" else "weights_bf16")
+
+
+@pytest.mark.gpu
+def test_phase_ranges_change_nothing(tiny_models):
+    """EngineConfig.trace_ranges marks schedule / prepare / forward / sample of every step for a profiler (the
+    reference marks the same phases, inference_engine/engine.py:183-210); with or without them the same tokens."""
+    m = tiny_models["A"]
+    prompts = prompts_for(m, [5, 17, 33], seed=3)
+    sp = SamplingParams(max_tokens=6, ignore_eos=True, temperature=0.7, seed=11)
+    outs = []
+    for ranges in (False, True):
+        eng = engine(m, "cuda", "float32", num_blocks=16, max_num_seqs=4, trace_ranges=ranges)
+        assert eng.runner.ranges.on == ranges
+        outs.append([o.output_ids for o in eng.generate(prompts, sp)])
+    assert outs[0] == outs[1]
