@@ -24,7 +24,8 @@ class EngineConfig:
     num_blocks: int | None = None           # explicit page count (scratch page included)
     num_state_slots: int | None = None      # default: max_num_seqs + 1 (slot 0 is scratch)
     use_hip_graphs: bool = True
-    graph_batch_sizes: tuple = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 160, 192, 224, 256)
+    # up to 16 rows a step's time grows with every row (13 us a row at TinyLlama sizes), from 17 to 32 hardly: hence 6 and 12
+    graph_batch_sizes: tuple = (1, 2, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 160, 192, 224, 256)
     portion_graph_sizes: tuple | None = None   # token counts of the captured single-prompt steps; None: eighths of the token budget
     seed: int = 0                           # base of every request's sampling stream
     activation_reserve_bytes: int = 768 * 2**20
